@@ -24,12 +24,14 @@ from .state import StateSlots
 
 @dataclass(frozen=True)
 class CacheGroup:
-    """Cache slots that keep the same planes per token over the same window (0: every token)."""
+    """Cache slots that keep the same planes per token over the same window (0: every token; with a window,
+    ``keep_first`` tokens at the start of the sequence stay as well)."""
 
     index: int
     planes: tuple  # of parts.base.CachePlane: name, heads, width, token_minor
     window: int
     slots: tuple[int, ...]
+    keep_first: int = 0
 
     @property
     def elements_per_token(self) -> int:
@@ -58,13 +60,14 @@ class CacheLayout:
         states = []
         for n in needs:
             if n.kv is not None:
-                key = (tuple((p.name, p.heads, p.width, p.token_minor) for p in n.kv.planes), n.kv.window)
+                key = (tuple((p.name, p.heads, p.width, p.token_minor) for p in n.kv.planes), n.kv.window,
+                       getattr(n.kv, "keep_first", 0))
                 by_key.setdefault(key, []).append(n.slot)
                 planes_of[key] = tuple(n.kv.planes)
             if n.state is not None:
                 states.append(StateGroup(n.slot, tuple(n.state.tensors)))
         groups = tuple(
-            CacheGroup(i, planes_of[key], key[1], tuple(slots)) for i, (key, slots) in enumerate(sorted(by_key.items()))
+            CacheGroup(i, planes_of[key], key[1], tuple(slots), key[2]) for i, (key, slots) in enumerate(sorted(by_key.items()))
         )
         return cls(groups, tuple(states), {s: g.index for g in groups for s in g.slots})
 
@@ -115,6 +118,10 @@ class CacheManager:
     def pages(self, n_tokens: int) -> int:
         return -(-n_tokens // self.page_size)
 
+    def keep_pages(self, group: CacheGroup) -> int:
+        """Pages at the start of a sequence that a windowed group never gives back."""
+        return self.pages(group.keep_first) if group.window else 0
+
     def free_pages(self) -> list[int]:
         return [a.num_free for a in self.allocators]
 
@@ -123,13 +130,14 @@ class CacheManager:
 
     def peak_pages(self, total_tokens: int, step_tokens: int | None = None) -> list[int]:
         """Most pages per group a request holds at any time on its way to ``total_tokens``, fed in
-        steps of at most ``step_tokens`` tokens. A windowed group needs the window plus one step."""
+        steps of at most ``step_tokens`` tokens. A windowed group needs the window plus one step (and the
+        first pages it keeps)."""
         step = step_tokens if step_tokens else self.max_step_tokens
         out = []
         for g in self.layout.groups:
             full = self.pages(total_tokens)
             if g.window and step:
-                full = min(full, self.pages(g.window - 1 + step) + 1)
+                full = min(full, self.pages(g.window - 1 + step) + 1 + self.keep_pages(g))
             out.append(full)
         return out
 
@@ -181,11 +189,12 @@ class CacheManager:
 
     def advance(self, rc: RequestCache) -> int:
         """After a step: give back the pages of windowed groups that no later query can see
-        (a query at position p >= num_tokens sees keys from p - window + 1 on). Returns how many."""
+        (a query at position p >= num_tokens sees keys from p - window + 1 on, and the group's kept first
+        tokens). Returns how many."""
         freed = 0
         for g, t in zip(self.layout.groups, rc.tables):
             if g.window:
-                freed += t.release_before(rc.num_tokens - g.window + 1)
+                freed += t.release_before(rc.num_tokens - g.window + 1, self.keep_pages(g))
         return freed
 
     def release(self, rc: RequestCache) -> None:

@@ -31,7 +31,8 @@ def _library():
             "msb_table_num_tokens": ([_P], _I), "msb_table_num_blocks": ([_P], _I), "msb_table_first_live": ([_P], _I),
             "msb_table_blocks_needed": ([_P, _I], _I), "msb_table_append": ([_P, _I, _P, _I, _IP], _I),
             "msb_table_slot": ([_P, _I, _IP], _I), "msb_table_tail_slots": ([_P, _I, _P], _I),
-            "msb_table_rewind": ([_P, _I], _I), "msb_table_release_before": ([_P, _I, _IP], _I),
+            "msb_table_rewind": ([_P, _I], _I), "msb_table_release_before": ([_P, _I, _I, _IP], _I),
+            "msb_table_kept": ([_P], _I),
             "msb_table_release": ([_P], _I), "msb_table_blocks": ([_P, _P, _I], _I),
             "msb_pack_tables": ([_P, _I, _P, _I, _I, _I, _I, _IP], _I),
         }
@@ -142,8 +143,12 @@ class NativePageTable:
         return self._lib.msb_table_first_live(self._h)
 
     @property
+    def kept(self) -> int:
+        return self._lib.msb_table_kept(self._h)
+
+    @property
     def num_held(self) -> int:
-        return self.num_entries - self.first_live
+        return self.num_entries - self.first_live + self.kept
 
     @property
     def entries(self) -> np.ndarray:
@@ -187,9 +192,11 @@ class NativePageTable:
     def rewind(self, n: int) -> None:
         _raise(self._lib.msb_table_rewind(self._h, n), f"cannot rewind {n} tokens")
 
-    def release_before(self, pos: int) -> int:
+    def release_before(self, pos: int, keep_pages: int = 0) -> int:
+        if keep_pages < 0:
+            raise ValueError(f"cannot keep {keep_pages} pages")
         out = _I()
-        _raise(self._lib.msb_table_release_before(self._h, pos, ctypes.byref(out)), "release_before")
+        _raise(self._lib.msb_table_release_before(self._h, pos, keep_pages, ctypes.byref(out)), "release_before")
         return out.value
 
     def release(self) -> None:

@@ -10,7 +10,9 @@ The order in which pages are handed out is a contract (the C++ core and the refe
 are checked id for id, miniserve/cache/block_allocator.py:24-107, block_table.py:19-89): a fresh
 group hands out 0, 1, 2, ...; pages given back are used again newest first; taking pages is all or
 nothing; giving back checks the whole call before anything changes. Beyond the reference: a table
-gives back the pages a window has passed (``release_before``); those entries read ``NO_PAGE``.
+gives back the pages a window has passed (``release_before``); those entries read ``NO_PAGE``. A window
+may keep the sequence's first tokens visible: ``release_before(pos, keep_pages)`` never gives back the
+first ``keep_pages`` entries.
 """
 
 from __future__ import annotations
@@ -132,7 +134,8 @@ class PageTable:
         self._entries = np.empty(max(8, int(shared.size)), dtype=np.int32)
         self._entries[: shared.size] = shared
         self.num_entries = int(shared.size)  # pages held plus entries already given back
-        self.first_live = 0  # index of the first entry that still holds a page
+        self.first_live = 0  # index of the first entry behind the gap that still holds a page
+        self.kept = 0  # entries before the gap that stay held (the kept first pages of a window)
         self.num_tokens = self.num_entries * self.page_size  # a shared prefix is whole pages
 
     # -------------------------------------------------------------- views
@@ -147,7 +150,7 @@ class PageTable:
 
     @property
     def num_held(self) -> int:
-        return self.num_entries - self.first_live
+        return self.num_entries - self.first_live + self.kept
 
     # -------------------------------------------------------------- growth
 
@@ -211,20 +214,25 @@ class PageTable:
 
     # -------------------------------------------------------------- pages going back
 
-    def release_before(self, pos: int) -> int:
-        """Give back every page whose tokens all lie before ``pos``. Returns how many."""
+    def release_before(self, pos: int, keep_pages: int = 0) -> int:
+        """Give back every page whose tokens all lie before ``pos``, except the first ``keep_pages``
+        entries (the same number in every call for one table). Returns how many."""
+        if keep_pages < 0:
+            raise ValueError(f"cannot keep {keep_pages} pages")
         upto = min(max(pos, 0) // self.page_size, self.num_entries)
-        if upto <= self.first_live:
+        start = max(self.first_live, keep_pages)
+        if upto <= start:
             return 0
-        self.allocator.give_back(self._entries[self.first_live : upto])
-        self._entries[self.first_live : upto] = NO_PAGE
-        gone = upto - self.first_live
+        self.allocator.give_back(self._entries[start:upto])
+        self._entries[start:upto] = NO_PAGE
+        if self.first_live <= keep_pages:
+            self.kept = keep_pages
         self.first_live = upto
-        return gone
+        return upto - start
 
     def release(self) -> None:
-        self.allocator.give_back(self._entries[self.first_live : self.num_entries])
-        self.num_entries = self.num_tokens = self.first_live = 0
+        self.allocator.give_back(np.concatenate((self._entries[: self.kept], self._entries[self.first_live : self.num_entries])))
+        self.num_entries = self.num_tokens = self.first_live = self.kept = 0
 
 
 def pack_tables(tables, out: np.ndarray, pad_rows: int = 0, pad_page: int = 0) -> int:

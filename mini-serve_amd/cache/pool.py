@@ -35,6 +35,7 @@ class LayerCache:
     writes: bool
     page_size: int
     window: int
+    keep_first: int = 0  # with a window: the sequence's first tokens that stay visible
 
     @property
     def k(self) -> torch.Tensor:
@@ -87,7 +88,8 @@ class KVPool:
         gi, i = where
         gb = batch.groups[gi]
         planes = {name: buf[i] for name, buf in self.buffers[gi].items()}
-        return LayerCache(planes, gb.block_table, gb.slots, writes, self.page_size, self.layout.groups[gi].window)
+        g = self.layout.groups[gi]
+        return LayerCache(planes, gb.block_table, gb.slots, writes, self.page_size, g.window, g.keep_first)
 
     def state_view(self, slot: int, batch) -> dict | None:
         """The state tensors of a cache slot by name (None if its mixer keeps none); row

@@ -56,10 +56,13 @@ def load_config_dict(path: str | Path) -> dict:
 
 
 def architecture_name(cfg: dict) -> str:
+    """The name under ``architectures`` (a list, its first entry) or ``architecture`` (a string)."""
     archs = cfg.get("architectures")
+    if archs is None and isinstance(cfg.get("architecture"), str):
+        return cfg["architecture"]
     if not archs or not isinstance(archs, (list, tuple)) or not isinstance(archs[0], str):
         raise ValueError(
-            f"config.json names no architecture (key 'architectures'); known: {sorted(ARCHITECTURES)}"
+            f"config.json names no architecture (key 'architectures' or 'architecture'); known: {sorted(ARCHITECTURES)}"
         )
     return archs[0]
 

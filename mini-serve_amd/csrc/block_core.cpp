@@ -81,6 +81,7 @@ struct Table {
   std::vector<int> blocks;
   int num_tokens = 0;
   int first_live = 0;
+  int kept = 0;  // entries before the gap that stay held: the first pages a window keeps
 
   int needed(int n) const {
     const int bs = alloc->block_size;
@@ -120,24 +121,31 @@ struct Table {
     num_tokens -= n;
     return OK;
   }
-  int release_before(int pos, int* freed) {
+  // Gives back every block whose tokens all lie before pos, except the first `keep` entries.
+  int release_before(int pos, int keep, int* freed) {
+    if (keep < 0) return BAD_ARG;
     int upto = (pos > 0 ? pos : 0) / alloc->block_size;
     if (upto > (int)blocks.size()) upto = (int)blocks.size();
     *freed = 0;
-    if (upto <= first_live) return OK;
-    const int st = alloc->release(blocks.data() + first_live, upto - first_live);
+    const int start = first_live > keep ? first_live : keep;
+    if (upto <= start) return OK;
+    const int st = alloc->release(blocks.data() + start, upto - start);
     if (st != OK) return st;
-    for (int i = first_live; i < upto; ++i) blocks[i] = NO_BLOCK;
-    *freed = upto - first_live;
+    for (int i = start; i < upto; ++i) blocks[i] = NO_BLOCK;
+    *freed = upto - start;
+    if (first_live <= keep) kept = keep;
     first_live = upto;
     return OK;
   }
   int release_all() {
-    const int st = alloc->release(blocks.data() + first_live, (int)blocks.size() - first_live);
+    std::vector<int> held(blocks.begin(), blocks.begin() + kept);
+    held.insert(held.end(), blocks.begin() + first_live, blocks.end());
+    const int st = alloc->release(held.data(), (int)held.size());
     if (st != OK) return st;
     blocks.clear();
     num_tokens = 0;
     first_live = 0;
+    kept = 0;
     return OK;
   }
 };
@@ -172,7 +180,7 @@ void* msb_table_new(void* a, const int* prefix, int n, int* status) {
   }
   *status = al->incref(prefix, n);
   if (*status != OK) return nullptr;
-  auto* t = new Table{al, {}, 0, 0};
+  auto* t = new Table{al, {}, 0, 0, 0};
   t->blocks.assign(prefix, prefix + n);
   t->num_tokens = n * al->block_size;
   return t;
@@ -188,7 +196,10 @@ int msb_table_append(void* t, int n, int* fresh, int cap, int* n_fresh) {
 int msb_table_slot(void* t, int pos, int* out) { return static_cast<Table*>(t)->slot(pos, out); }
 int msb_table_tail_slots(void* t, int n, int* out) { return static_cast<Table*>(t)->tail_slots(n, out); }
 int msb_table_rewind(void* t, int n) { return static_cast<Table*>(t)->rewind(n); }
-int msb_table_release_before(void* t, int pos, int* freed) { return static_cast<Table*>(t)->release_before(pos, freed); }
+int msb_table_kept(void* t) { return static_cast<Table*>(t)->kept; }
+int msb_table_release_before(void* t, int pos, int keep, int* freed) {
+  return static_cast<Table*>(t)->release_before(pos, keep, freed);
+}
 int msb_table_release(void* t) { return static_cast<Table*>(t)->release_all(); }
 int msb_table_blocks(void* t, int* out, int cap) {
   auto* tb = static_cast<Table*>(t);

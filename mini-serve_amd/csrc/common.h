@@ -83,10 +83,23 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ p, int spl
 // Activations of the gated feed-forward, by the number the host passes: out = act(gate) * up, in float32.
 #define MS_ACT_SILU 0
 #define MS_ACT_GELU_TANH 1
-#define MS_ACT_COUNT 2
+#define MS_ACT_COUNT 2  // the activations of the form act(gate) * up, which the matrix kernels' epilogues know
+// A gated feed-forward with bounded inputs: g = min(gate, limit), u = clamp(up, -limit, limit),
+// out = g sigmoid(1.702 g) (u + 1). Not of the form act(gate) * up: it takes `limit` beside the number.
+#define MS_ACT_SWIGLU_CLAMPED 2
+#define MS_GATED_COUNT 3
 __device__ __forceinline__ float activate(float x, int act) {
   if (act == MS_ACT_GELU_TANH) return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
   return x / (1.f + expf(-x));
+}
+// What a gated feed-forward makes of one gate and one up value, float32.
+__device__ __forceinline__ float gated_value(float gate, float up, int act, float limit) {
+  if (act == MS_ACT_SWIGLU_CLAMPED) {
+    const float g = fminf(gate, limit);
+    const float u = fminf(fmaxf(up, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return activate(gate, act) * up;
 }
 
 static inline int launch_status() { return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED; }

@@ -237,30 +237,30 @@ __device__ __forceinline__ int gate_at(int i, int block) { return block ? (i / b
 __device__ __forceinline__ int up_at(int i, int inter, int block) { return block ? gate_at(i, block) + block : inter + i; }
 
 template <typename T>
-__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int block, int act) {
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int block, int act, float limit) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const float g = to_f32(gu[(size_t)t * 2 * inter + gate_at(i, block)]);
   const float u = to_f32(gu[(size_t)t * 2 * inter + up_at(i, inter, block)]);
-  out[(size_t)t * inter + i] = from_f32<T>(activate(g, act) * u);
+  out[(size_t)t * inter + i] = from_f32<T>(gated_value(g, u, act, limit));
 }
 
 // The same with gu given as float partial sums [splits, tokens, 2 * inter] (summed in ascending order).
 template <typename T>
 __global__ void act_mul_parts_kernel(const float* __restrict__ parts, int splits, size_t split_stride,
-                                     T* __restrict__ out, int inter, int block, int act) {
+                                     T* __restrict__ out, int inter, int block, int act, float limit) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= inter) return;
   const float* row = parts + (size_t)t * 2 * inter;
   const float g = sum_splits(row + gate_at(i, block), splits, split_stride);
   const float u = sum_splits(row + up_at(i, inter, block), splits, split_stride);
-  out[(size_t)t * inter + i] = from_f32<T>(activate(g, act) * u);
+  out[(size_t)t * inter + i] = from_f32<T>(gated_value(g, u, act, limit));
 }
 
 // bfloat16 with inter (and block) a multiple of 8: eight elements per thread, moved as 16-byte vectors.
-__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int inter, int block, int act) {
+__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int inter, int block, int act, float limit) {
   const int t = blockIdx.y;
   const int i = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (i >= inter) return;
@@ -270,30 +270,35 @@ __global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restric
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float gv = to_f32(g.e[e]);
-    o.e[e] = from_f32<bf16>(activate(gv, act) * to_f32(u.e[e]));
+    o.e[e] = from_f32<bf16>(gated_value(gv, to_f32(u.e[e]), act, limit));
   }
   *reinterpret_cast<uint4*>(out + (size_t)t * inter + i) = o.u;
 }
 
-extern "C" int ms_act_mul(const void* gu, void* out, int is_bf16, int tokens, int inter, int block, int act, hipStream_t st) {
+// act: an MS_ACT_* number below MS_GATED_COUNT; limit: the bound of MS_ACT_SWIGLU_CLAMPED (ignored by the others).
+extern "C" int ms_act_mul(const void* gu, void* out, int is_bf16, int tokens, int inter, int block, int act, float limit,
+                          hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (inter <= 0 || tokens > 65535 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_ACT_COUNT) return MS_BAD_ARG;
+  if (inter <= 0 || tokens > 65535 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_GATED_COUNT ||
+      (act == MS_ACT_SWIGLU_CLAMPED && !(limit > 0.f)))
+    return MS_BAD_ARG;
   dim3 grid((inter + 255) / 256, tokens);
   if (is_bf16 && inter % 8 == 0 && block % 8 == 0)
-    act_mul_vec8_kernel<<<dim3((inter / 8 + 255) / 256, tokens), 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act);
-  else if (is_bf16) act_mul_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act);
-  else act_mul_kernel<float><<<grid, 256, 0, st>>>((const float*)gu, (float*)out, inter, block, act);
+    act_mul_vec8_kernel<<<dim3((inter / 8 + 255) / 256, tokens), 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act, limit);
+  else if (is_bf16) act_mul_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)gu, (bf16*)out, inter, block, act, limit);
+  else act_mul_kernel<float><<<grid, 256, 0, st>>>((const float*)gu, (float*)out, inter, block, act, limit);
   return launch_status();
 }
 
 extern "C" int ms_act_mul_parts(const float* parts, int splits, long long split_stride, void* out, int out_is_bf16,
-                                int tokens, int inter, int block, int act, hipStream_t st) {
+                                int tokens, int inter, int block, int act, float limit, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (inter <= 0 || tokens > 65535 || splits < 1 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_ACT_COUNT)
+  if (inter <= 0 || tokens > 65535 || splits < 1 || block < 0 || (block > 0 && inter % block) || act < 0 || act >= MS_GATED_COUNT ||
+      (act == MS_ACT_SWIGLU_CLAMPED && !(limit > 0.f)))
     return MS_BAD_ARG;
   dim3 grid((inter + 255) / 256, tokens);
-  if (out_is_bf16) act_mul_parts_kernel<bf16><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (bf16*)out, inter, block, act);
-  else act_mul_parts_kernel<float><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (float*)out, inter, block, act);
+  if (out_is_bf16) act_mul_parts_kernel<bf16><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (bf16*)out, inter, block, act, limit);
+  else act_mul_parts_kernel<float><<<grid, 256, 0, st>>>(parts, splits, (size_t)split_stride, (float*)out, inter, block, act, limit);
   return launch_status();
 }
 

@@ -58,7 +58,8 @@ class ModelRunner:
         graph_rows = (decode_graph_max_bs or max_running) if decode_graph else 0
         # What a windowed group needs at most: per running request the window, one step, and a page's slack.
         self.window_pages = [
-            max_running * (-(-(g.window - 1 + request_step_tokens) // page_size) + 1) if g.window and request_step_tokens else None
+            max_running * (-(-(g.window - 1 + request_step_tokens) // page_size) + 1 + -(-g.keep_first // page_size))
+            if g.window and request_step_tokens else None
             for g in self.layout.groups
         ]
         self.kv_profile = {"page_size": page_size, "bytes_per_page": per_page, "kv_mem_fraction": kv_mem_fraction}

@@ -24,8 +24,17 @@ _SIGNATURES = {
     "ms_embed": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
     "ms_feed_tokens": [_c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     "ms_rmsnorm": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int, _c_ll, _c_void],
-    "ms_act_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_act_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_act_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
+    "ms_act_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
+    "ms_layernorm": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
+    "ms_group_rmsnorm_gate": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
+    "ms_normed_mean_add": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void],
+    "ms_scale": [_c_void, _c_ll, _c_float, _c_void],
+    "ms_qkv_norm_rope_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int, _c_int,
+                               _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_gated_recurrence": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                            _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                            _c_int, _c_void],
     "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
     "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -41,7 +50,7 @@ _SIGNATURES = {
     "ms_gemm_bf16_small_tile_cols": [_c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
-                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
+                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void,
@@ -247,21 +256,29 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 
 # Activations of the gated feed-forward and the numbers the kernels know them by (MS_ACT_* in csrc/common.h):
 # silu(x) = x sigmoid(x); gelu_tanh(x) = x / 2 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))).
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+# swiglu_clamped(gate, up) = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit): not of
+# the form act(gate) * up, it takes ``limit`` along and runs in the activation kernels (no matrix kernel's epilogue knows it).
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swiglu_clamped": 2}
+ACTIVATIONS_WITH_LIMIT = {"swiglu_clamped"}
 
 
-def _activation(name: str) -> int:
+def _activation(name: str, limit: float | None = None) -> int:
     try:
-        return ACTIVATIONS[name]
+        act = ACTIVATIONS[name]
     except KeyError:
         raise NotImplementedError(f"activation {name!r}: the kernels know {sorted(ACTIVATIONS)}") from None
+    if name in ACTIVATIONS_WITH_LIMIT and not (limit is not None and limit > 0):
+        raise ValueError(f"activation {name!r} needs a positive limit, got {limit!r}")
+    return act
 
 
-def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> torch.Tensor:
-    """``act(gate) * up`` for ``gu [T, 2 I]``, a tensor or a ``SplitSum`` (then ``out_dtype`` names the
+def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0, limit: float | None = None) -> torch.Tensor:
+    """``act(gate) * up`` (or what ``activation`` makes of gate and up) for ``gu [T, 2 I]``, a tensor or a
+    ``SplitSum`` (then ``out_dtype`` names the
     result's dtype). ``block == 0``: the row holds the ``I`` gates, then the ``I`` ups; ``block > 0``:
     alternating runs of ``block`` gates and ``block`` ups (see ``interleave_gate_up``)."""
-    act = _activation(activation)
+    act = _activation(activation, limit)
+    limit = float(limit or 0.0)
     if isinstance(gu, SplitSum):
         _dev(gu.parts, "gu", F32, 3)
         t, width = gu.shape
@@ -271,7 +288,7 @@ def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> tor
         for t0 in range(0, t, 32768):
             n = min(32768, t - t0)
             _check(library().ms_act_mul_parts(gu.parts[:, t0:].data_ptr(), gu.splits, gu.stride, out[t0:].data_ptr(),
-                                              int(out_dtype == BF16), n, width // 2, int(block), act, _stream()), "act_mul")
+                                              int(out_dtype == BF16), n, width // 2, int(block), act, limit, _stream()), "act_mul")
         return out
     _dev(gu, "gu", (F32, BF16), 2)
     if gu.shape[1] % 2 or (block and (gu.shape[1] // 2) % block):
@@ -281,24 +298,25 @@ def act_mul(gu, activation: str = "silu", out_dtype=None, block: int = 0) -> tor
     # grid.y carries the token index: split very long batches
     for t0 in range(0, gu.shape[0], 32768):
         n = min(32768, gu.shape[0] - t0)
-        _check(library().ms_act_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, int(block), act,
+        _check(library().ms_act_mul(gu[t0:].data_ptr(), out[t0:].data_ptr(), int(gu.dtype == BF16), n, inter, int(block), act, limit,
                                     _stream()), "act_mul")
     return out
 
 
-def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu", out_dtype=None, block: int = 0):
+def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu", out_dtype=None, block: int = 0,
+                 limit: float | None = None):
     """``act(x gate^T) * (x up^T)`` for ``gate_up [2 I, K]`` laid out as ``act_mul`` describes. With
     interleaved bfloat16 weights the activation runs in the matrix kernel's epilogue where a kernel
     for the shape exists (few rows: no partial sums leave the kernel; many rows: the gate/up matrix is
     never written); otherwise the product and the activation are two kernels."""
-    act = _activation(activation)
+    act = _activation(activation, limit)
     _dev(x, "x", (F32, BF16), 2)
     _dev(gate_up, "gate_up", (F32, BF16), 2)
     m, k = x.shape
     if gate_up.shape[1] != k or gate_up.shape[0] % 2:
         raise ValueError(f"gated_linear: x is [{m}, {k}], gate_up is {tuple(gate_up.shape)}")
     inter = gate_up.shape[0] // 2
-    if block == GATE_BLOCK and gate_up.dtype == BF16 and out_dtype == BF16 and m > 0:
+    if block == GATE_BLOCK and gate_up.dtype == BF16 and out_dtype == BF16 and m > 0 and activation not in ACTIVATIONS_WITH_LIMIT:
         xa = cast(x, BF16)
         out = torch.empty((m, inter), dtype=BF16, device=x.device)
         rc = library().ms_gemm_bf16_gated(xa.data_ptr(), gate_up.data_ptr(), out.data_ptr(), m, inter, k, k, act, _stream())
@@ -307,7 +325,7 @@ def gated_linear(x: torch.Tensor, gate_up: torch.Tensor, activation: str = "silu
         if rc != 2:  # 2: no fused kernel for this shape
             _check(rc, "gemm_bf16_gated")
     gu = linear(x, gate_up, out_dtype=out_dtype, defer=True)
-    return act_mul(gu, activation, out_dtype=out_dtype, block=block)
+    return act_mul(gu, activation, out_dtype=out_dtype, block=block, limit=limit)
 
 
 def cast(x: torch.Tensor, dtype) -> torch.Tensor:
@@ -492,15 +510,17 @@ def qk_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cac
     return q_out
 
 
-def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim) -> int:
-    """Keys ``[pages, Hkv, page, D]``, values ``[pages, Hkv, D, page]``; returns the page size."""
+def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, value_dim: int | None = None) -> int:
+    """Keys ``[pages, Hkv, page, D]``, values ``[pages, Hkv, Dv, page]`` (``Dv = D`` unless ``value_dim`` is
+    given); returns the page size."""
     _dev(k_cache, "k_cache", dtype, 4)
     _dev(v_cache, "v_cache", dtype, 4)
     page = k_cache.shape[2]
+    dv = head_dim if value_dim is None else value_dim
     if tuple(k_cache.shape[1:]) != (num_kv_heads, page, head_dim):
         raise ValueError(f"k_cache is {tuple(k_cache.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
-    if tuple(v_cache.shape) != (k_cache.shape[0], num_kv_heads, head_dim, page):
-        raise ValueError(f"v_cache is {tuple(v_cache.shape)}, expected [{k_cache.shape[0]}, {num_kv_heads}, {head_dim}, {page}]")
+    if tuple(v_cache.shape) != (k_cache.shape[0], num_kv_heads, dv, page):
+        raise ValueError(f"v_cache is {tuple(v_cache.shape)}, expected [{k_cache.shape[0]}, {num_kv_heads}, {dv}, {page}]")
     return page
 
 
@@ -600,18 +620,25 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
     return SplitSum(merged)
 
 
-def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window):
+def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window,
+                    value_dim: int | None = None, keep_first: int = 0, exact_weights: bool = False):
     """Attention of the batch's new tokens over the cache. ``qkv [T, >= Hq D]`` holds the queries
-    in its first ``Hq * D`` columns. Returns ``[T, Hq * D]``.
+    in its first ``Hq * D`` columns. Returns ``[T, Hq * Dv]`` (``Dv = D`` unless ``value_dim`` is given).
+    A query at position p sees keys ``max(0, p - window + 1) .. p`` (``window == 0``: all up to p) and, with a
+    window, the keys ``0 .. keep_first - 1`` as well.
 
     bfloat16 with 16-token pages and a head size of 64 or 128: rows that bring one token run the
     split decode kernel, rows that bring several the tiled prefill kernel. Everything else (float32,
-    other head sizes or page sizes) runs the generic kernel."""
+    other head sizes or page sizes, values of another size than the keys, kept first keys, or
+    ``exact_weights``: softmax weights that must meet the values unrounded) runs the generic kernel."""
     _dev(qkv, "qkv", (F32, BF16), 2)
     t = qkv.shape[0]
-    page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim)
-    if head_dim % 16 or not 16 <= head_dim <= 256:
-        raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 up to 256")
+    dv = head_dim if value_dim is None else int(value_dim)
+    page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, dv)
+    if not (1 <= head_dim <= 256 and 1 <= dv <= 256):
+        raise ValueError(f"head sizes {head_dim} / {dv} are not supported: the attention kernels take sizes up to 256")
+    if keep_first < 0 or window < 0:
+        raise ValueError("window and keep_first must not be negative")
     if num_heads % num_kv_heads:
         raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} KV heads")
     if qkv.shape[1] < num_heads * head_dim:
@@ -623,17 +650,18 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     _dev(batch.positions, "positions", I32, 1)
     if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
         raise ValueError("batch metadata does not match the number of tokens or rows")
-    out = torch.empty((t, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    out = torch.empty((t, num_heads * dv), dtype=qkv.dtype, device=qkv.device)
     lib = library()
     common = (block_table.data_ptr(), block_table.shape[1])
     meta = (batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr())
     n_dec = batch.num_decode_tokens
     fast = (qkv.dtype == BF16 and page == 16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 16
-            and qkv.shape[1] % 8 == 0)
+            and qkv.shape[1] % 8 == 0 and dv == head_dim and not (window and keep_first) and not exact_weights)
     if not fast:
         _check(lib.ms_paged_attention_generic(
             qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common, None,
-            *meta, t, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()), "paged_attention")
+            *meta, t, num_heads, num_kv_heads, head_dim, dv, page, float(scale), int(window), int(keep_first), _stream()),
+            "paged_attention")
         return out
     if n_dec:
         splits = decode_splits(n_dec, num_kv_heads, batch.max_kv_len)
@@ -772,6 +800,205 @@ def _prefill_parts_plan(batch, tile_tokens: int, kv_heads: int, part_bytes: int)
         memo[key] = plan
     return plan
 
+
+
+# ------------------------------------------------------------------------------------- further norms
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, eps: float, out_dtype,
+              rows: torch.Tensor | None = None) -> torch.Tensor:
+    """``(x - mean) / sqrt(var + eps) * weight + bias`` over the float32 rows of ``x`` (all, or those named by
+    ``rows``), statistics in float32, the variance being the mean of the squared deviations."""
+    _dev(x, "x", F32, 2)
+    _dev(weight, "weight", (F32, BF16), 1)
+    if weight.shape[0] != x.shape[1]:
+        raise ValueError(f"norm weight has {weight.shape[0]} elements for width {x.shape[1]}")
+    if bias is not None:
+        _dev(bias, "bias", weight.dtype, 1)
+        if bias.shape[0] != x.shape[1]:
+            raise ValueError(f"norm bias has {bias.shape[0]} elements for width {x.shape[1]}")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    n = x.shape[0]
+    if rows is not None:
+        _dev(rows, "rows", I32, 1)
+        n = rows.shape[0]
+    out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+    _check(library().ms_layernorm(x.data_ptr(), weight.data_ptr(), _ptr(bias), int(weight.dtype == BF16), out.data_ptr(),
+                                  int(out_dtype == BF16), _ptr(rows), n, x.shape[1], float(eps), _stream()), "layernorm")
+    return out
+
+
+def group_rmsnorm_gate(x: torch.Tensor, group: int, weight: torch.Tensor | None, gate: torch.Tensor | None, eps: float,
+                       out_dtype) -> torch.Tensor:
+    """``x / rms(group of x) * weight * sigmoid(gate)`` for float32 ``x [T, N]`` cut into groups of ``group``
+    consecutive elements (``group == N``: one norm over the row). ``weight [N]`` and ``gate`` (float32 ``[T, N]``,
+    may be a column slice of a wider matrix) are optional."""
+    _dev(x, "x", F32, 2)
+    t, n = x.shape
+    if group < 1 or n % group:
+        raise ValueError(f"a row of {n} elements cannot be cut into groups of {group}")
+    if weight is not None:
+        _dev(weight, "weight", (F32, BF16), 1)
+        if weight.shape[0] != n:
+            raise ValueError(f"norm weight has {weight.shape[0]} elements for width {n}")
+    gate_stride = 0
+    if gate is not None:
+        if not (gate.is_cuda and gate.dtype == F32 and gate.dim() == 2 and gate.shape == x.shape and gate.stride(1) == 1):
+            raise ValueError("gate must be a float32 matrix of x's shape on the GPU with unit column stride")
+        gate_stride = gate.stride(0)
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    out = torch.empty((t, n), dtype=out_dtype, device=x.device)
+    _check(library().ms_group_rmsnorm_gate(x.data_ptr(), _ptr(weight), int(weight is not None and weight.dtype == BF16), _ptr(gate),
+                                           gate_stride, out.data_ptr(), int(out_dtype == BF16), t, n // group, group, float(eps),
+                                           _stream()), "group_rmsnorm_gate")
+    return out
+
+
+def normed_mean_add(residual: torch.Tensor, streams, weights, eps: float, coef: float) -> None:
+    """``residual += coef * sum_i rmsnorm(streams[i]) * weights[i]``: up to four float32 streams of the residual's
+    shape, each normed over the row with its own weight."""
+    _dev(residual, "residual", F32, 2)
+    n = len(streams)
+    if not 1 <= n <= 4 or len(weights) != n:
+        raise ValueError("one to four streams, each with a weight, are needed")
+    for s_, w in zip(streams, weights):
+        _dev(s_, "stream", F32, 2)
+        _dev(w, "weight", weights[0].dtype, 1)
+        if s_.shape != residual.shape or w.shape[0] != residual.shape[1]:
+            raise ValueError("streams and weights must have the residual's shape and width")
+    _dev(weights[0], "weight", (F32, BF16), 1)
+    sp = (ctypes.c_void_p * n)(*[s_.data_ptr() for s_ in streams])
+    wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+    _check(library().ms_normed_mean_add(residual.data_ptr(), sp, wp, int(weights[0].dtype == BF16), n, residual.shape[0],
+                                        residual.shape[1], float(eps), float(coef), _stream()), "normed_mean_add")
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` in place (float32)."""
+    _dev(x, "x", F32)
+    _check(library().ms_scale(x.data_ptr(), x.numel(), float(factor), _stream()), "scale")
+    return x
+
+
+def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
+                        value_dim, out_dtype, pairing: str = "halves") -> torch.Tensor:
+    """From float32 ``qkv [T, Hq D + Hkv D + Hkv Dv]``: RMS norm of the whole query part and of the whole key
+    part of a token (weights ``[Hq D]`` and ``[Hkv D]``; None: no norm), rotation of the first ``rope.shape[1]``
+    elements of each query and key head, in pairs as ``pairing`` names them, by the angles of ``rope`` (a
+    ``rope_table`` of these tokens; None: no rotation), keys and values stored into the cache pages at ``slots``
+    (skipped when ``slots`` is None). Returns the finished queries ``[T, Hq D]`` in ``out_dtype``."""
+    _dev(qkv, "qkv", F32, 2)
+    t = qkv.shape[0]
+    width = num_heads * head_dim + num_kv_heads * (head_dim + value_dim)
+    if qkv.shape[1] != width:
+        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    w_bf16 = 0
+    if (q_weight is None) != (k_weight is None):
+        raise ValueError("the query and the key norm come together or not at all")
+    if q_weight is not None:
+        for w, nm, n in ((q_weight, "q_norm", num_heads * head_dim), (k_weight, "k_norm", num_kv_heads * head_dim)):
+            _dev(w, nm, (F32, BF16), 1)
+            if w.shape[0] != n:
+                raise ValueError(f"{nm} weight has {w.shape[0]} elements, expected {n}")
+        if q_weight.dtype != k_weight.dtype:
+            raise TypeError("q_norm and k_norm weights differ in dtype")
+        w_bf16 = int(q_weight.dtype == BF16)
+    page_size = 1
+    if slots is not None:
+        _dev(slots, "slots", I32, 1)
+        if slots.shape[0] != t:
+            raise ValueError("one slot per token is needed")
+        page_size = _check_caches(k_cache, v_cache, out_dtype, num_kv_heads, head_dim, value_dim)
+    rot_dim, pair = 0, _pairing(pairing)
+    if rope is not None:
+        _dev(rope, "rope", F32, 2)
+        rot_dim = rope.shape[1]
+        if rope.shape[0] != t or rot_dim % 2 or rot_dim > head_dim or rot_dim < 2:
+            raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
+    q_out = torch.empty((t, num_heads * head_dim), dtype=out_dtype, device=qkv.device)
+    _check(library().ms_qkv_norm_rope_store(
+        qkv.data_ptr(), qkv.shape[1], q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
+        float(eps), _ptr(rope), int(rot_dim), pair, _ptr(k_cache) if slots is not None else None,
+        _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, int(value_dim), page_size, _stream()),
+        "qkv_norm_rope_store")
+    return q_out
+
+
+# ------------------------------------------------------------------------------------- linear recurrences
+
+RECURRENCE_MODES = {"decay": 0, "exp_gates": 1}
+RECURRENCE_MAX_DIM = 256
+
+
+def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
+                     mode: str, activation: str | None = None, q_scale: float = 1.0, decay: torch.Tensor | None = None,
+                     cap: float = 0.0, i_bias: torch.Tensor | None = None, f_bias: torch.Tensor | None = None) -> torch.Tensor:
+    """A linear recurrence over a matrix state per (request, head): ``S_t = a_t S_(t-1) + b_t k_t v_t^T``,
+    ``o_t = S_t^T q_t``, for the step's rows (``batch.row_start``, ``batch.starts``, ``batch.state_slots``), in float32.
+
+    ``x``: float32 ``[T, ld]`` whose columns hold the projections; ``columns``: first column of ``q`` and ``k``
+    (``heads * dim`` wide each), ``v`` (``heads * value_dim``) and, for ``mode="exp_gates"``, ``i`` and ``f`` (``heads``
+    each). ``activation`` (None or ``"silu"``) is applied to q, k and v; q is then scaled by ``q_scale``.
+    ``mode="decay"``: ``a = decay[head]``, ``b = 1``. ``mode="exp_gates"``: capped exponential gates with a running
+    maximum and a normaliser (the kernel's source states the formulas); ``state`` then also holds ``n`` and ``m``.
+    ``state["S"]``: float32 ``[slots, heads, dim, value_dim]``; rows with ``starts == 0`` begin from zero.
+    Returns float32 ``[T, heads * value_dim]``."""
+    _dev(x, "x", F32, 2)
+    t, ld = x.shape
+    if mode not in RECURRENCE_MODES:
+        raise NotImplementedError(f"recurrence mode {mode!r}: the kernels know {sorted(RECURRENCE_MODES)}")
+    if activation not in (None, "silu"):
+        raise NotImplementedError(f"activation {activation!r} inside the recurrence: None or 'silu'")
+    if dim > RECURRENCE_MAX_DIM or value_dim > RECURRENCE_MAX_DIM or min(dim, value_dim, heads) < 1:
+        raise ValueError(f"head sizes {dim} / {value_dim} are outside the recurrence kernels' range 1..{RECURRENCE_MAX_DIM}")
+    S = state["S"]
+    _dev(S, "S", F32, 4)
+    if tuple(S.shape[1:]) != (heads, dim, value_dim):
+        raise ValueError(f"state S is {tuple(S.shape)}, expected [slots, {heads}, {dim}, {value_dim}]")
+    n = m = None
+    if mode == "exp_gates":
+        n, m = state["n"], state["m"]
+        _dev(n, "n", F32, 3)
+        _dev(m, "m", F32, 2)
+        if tuple(n.shape) != (S.shape[0], heads, dim) or tuple(m.shape) != (S.shape[0], heads):
+            raise ValueError("state n / m do not match S")
+        if not cap > 0:
+            raise ValueError(f"the gates' cap must be positive, not {cap}")
+        for b_, nm in ((i_bias, "i_bias"), (f_bias, "f_bias")):
+            if b_ is not None:
+                _dev(b_, nm, (F32, BF16), 1)
+                if b_.shape[0] != heads:
+                    raise ValueError(f"{nm} has {b_.shape[0]} elements for {heads} heads")
+        if i_bias is not None and f_bias is not None and i_bias.dtype != f_bias.dtype:
+            raise TypeError("the gates' biases differ in dtype")
+    else:
+        _dev(decay, "decay", F32, 1)
+        if decay.shape[0] != heads:
+            raise ValueError(f"decay has {decay.shape[0]} elements for {heads} heads")
+    for name, w in (("q", heads * dim), ("k", heads * dim), ("v", heads * value_dim)) + (
+            (("i", heads), ("f", heads)) if mode == "exp_gates" else ()):
+        c = columns[name]
+        if c < 0 or c + w > ld:
+            raise ValueError(f"columns of {name!r} ({c} .. {c + w}) lie outside the matrix of width {ld}")
+    for v_, nm in ((batch.row_start, "row_start"), (batch.starts, "starts"), (batch.state_slots, "state_slots")):
+        _dev(v_, nm, I32, 1)
+    rows = batch.num_rows
+    if batch.row_start.shape[0] < rows + 1 or batch.starts.shape[0] < rows or batch.state_slots.shape[0] < rows:
+        raise ValueError("batch metadata does not match the number of rows")
+    if batch.num_tokens != t:
+        raise ValueError("one row of x per token of the step is needed")
+    out = torch.empty((t, heads * value_dim), dtype=F32, device=x.device)
+    bias = i_bias if i_bias is not None else f_bias
+    _check(library().ms_gated_recurrence(
+        x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], columns.get("i", 0), columns.get("f", 0), heads, dim, value_dim,
+        int(activation == "silu"), RECURRENCE_MODES[mode], float(q_scale), float(cap), _ptr(decay), _ptr(i_bias), _ptr(f_bias),
+        int(bias is not None and bias.dtype == BF16), S.data_ptr(), _ptr(n), _ptr(m), batch.row_start.data_ptr(),
+        batch.starts.data_ptr(), batch.state_slots.data_ptr(), out.data_ptr(), rows, _stream()), "gated_recurrence")
+    return out
 
 # ------------------------------------------------------------------------------------- sampling
 

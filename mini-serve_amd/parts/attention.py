@@ -12,6 +12,14 @@ for the next norm to add.
 
 ``window > 0`` restricts a query at position p to keys p-window+1 .. p (no counterpart in the
 reference). ``qk_norm_eps=None`` switches the per-head norms off; ``position`` may be ``none``.
+
+Further parameters, none of which the reference has (defaults give the layer above):
+``keep_first`` (with a window: the sequence's first ``keep_first`` keys stay visible at their true
+positions; the cache keeps their pages); ``value_dim`` (size of a value head, default ``head_dim``);
+``qk_norm="projection"`` (the RMS norm runs over a token's whole query projection and over its whole key
+projection, before they are split into heads, with weights of those sizes; default ``"head"``);
+``exact_weights`` (the softmax weights meet the values in float32: no rounding of them to bfloat16 for the
+matrix cores); ``names`` (the tensors' names behind the prefix, by ``q k v o q_norm k_norm``).
 """
 
 from __future__ import annotations
@@ -23,6 +31,14 @@ import torch
 from ..config.spec import PartSpec
 from .base import KVNeed, Mixer, TensorSpec
 from .registry import part_class, register
+
+
+def _names(spec: PartSpec) -> dict[str, str]:
+    p = spec.get("prefix", "")
+    given = spec.get("names") or {}
+    default = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+               "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+    return {k: p + given.get(k, d) for k, d in default.items()}
 
 
 @register("mixer", "gqa_attention")
@@ -37,14 +53,28 @@ class GQAttention(Mixer):
         self.scale = float(spec["scale"])
         self.qk_norm_eps = spec.get("qk_norm_eps")
         self.window = int(spec.get("window") or 0)
+        self.keep_first = int(spec.get("keep_first") or 0) if self.window else 0
+        self.value_dim = int(spec.get("value_dim") or self.head_dim)
+        self.qk_norm = spec.get("qk_norm", "head")
+        self.exact_weights = bool(spec.get("exact_weights", False))
+        self.names = _names(spec)
+        if self.qk_norm not in ("head", "projection"):
+            raise ValueError(f"qk_norm {self.qk_norm!r}: 'head' or 'projection'")
+        if self.keep_first < 0 or self.window < 0:
+            raise ValueError("window and keep_first must not be negative")
+        # The path with one norm over the projection, values of their own size, kept first keys or unrounded weights.
+        self.wide = (self.qk_norm == "projection" and self.qk_norm_eps is not None) or self.value_dim != self.head_dim
+        if self.wide and self.qk_norm == "head" and self.qk_norm_eps is not None:
+            raise NotImplementedError("a norm per head together with values of another size than the keys is not supported")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} query heads are no multiple of {self.kv_heads} KV heads")
         # What the attention kernels refuse is refused here, when the model is built, not in its first step.
-        if self.head_dim % 16 or not 16 <= self.head_dim <= 256:
-            raise ValueError(f"head_dim {self.head_dim} is not supported: the attention kernels take multiples of 16 from 16 to 256")
+        if not (1 <= self.head_dim <= 256 and 1 <= self.value_dim <= 256):
+            raise ValueError(f"head sizes {self.head_dim} / {self.value_dim} are not supported: the attention kernels take sizes up to 256")
         if not self.scale > 0:
             raise ValueError(f"the attention scale must be positive, not {self.scale}")
-        if rt is not None and rt.dtype == torch.bfloat16 and not (
+        generic = self.wide or self.exact_weights or self.keep_first
+        if rt is not None and rt.dtype == torch.bfloat16 and not generic and not (
                 self.head_dim in (64, 128) and self.heads // self.kv_heads <= 16):
             warnings.warn(
                 f"attention with head_dim {self.head_dim} and {self.heads // self.kv_heads} query heads per KV head runs the "
@@ -56,41 +86,52 @@ class GQAttention(Mixer):
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
-        p = spec.get("prefix", "")
+        n = _names(spec)
         h, d = int(spec["hidden_size"]), int(spec["head_dim"])
+        dv = int(spec.get("value_dim") or d)
         hq, hkv = int(spec["num_heads"]), int(spec["num_kv_heads"])
         out = {
-            p + "q_proj.weight": TensorSpec((hq * d, h)),
-            p + "k_proj.weight": TensorSpec((hkv * d, h)),
-            p + "v_proj.weight": TensorSpec((hkv * d, h)),
-            p + "o_proj.weight": TensorSpec((h, hq * d)),
+            n["q"]: TensorSpec((hq * d, h)),
+            n["k"]: TensorSpec((hkv * d, h)),
+            n["v"]: TensorSpec((hkv * dv, h)),
+            n["o"]: TensorSpec((h, hq * dv)),
         }
         if spec.get("qk_norm_eps") is not None:
-            out[p + "q_norm.weight"] = TensorSpec((d,), init="ones")
-            out[p + "k_norm.weight"] = TensorSpec((d,), init="ones")
+            whole = spec.get("qk_norm", "head") == "projection"
+            out[n["q_norm"]] = TensorSpec((hq * d if whole else d,), init="ones")
+            out[n["k_norm"]] = TensorSpec((hkv * d if whole else d,), init="ones")
         return out
 
     def bind(self, tensors) -> None:
-        p = self.prefix
-        parts = [tensors[p + n + "_proj.weight"] for n in ("q", "k", "v")]
+        p, n = self.prefix, self.names
+        parts = [tensors[n[k]] for k in ("q", "k", "v")]
         if len({t.dtype for t in parts}) != 1:
             raise ValueError(f"{p}q/k/v projections are stored in different dtypes")
         self.qkv = torch.cat(parts, dim=0).contiguous()
-        self.o = tensors[p + "o_proj.weight"]
+        self.o = tensors[n["o"]]
         if self.qk_norm_eps is not None:
-            self.q_norm = tensors[p + "q_norm.weight"]
-            self.k_norm = tensors[p + "k_norm.weight"]
+            self.q_norm = tensors[n["q_norm"]]
+            self.k_norm = tensors[n["k_norm"]]
 
     def kv_need(self) -> KVNeed:
-        return KVNeed.keys_values(self.kv_heads, self.head_dim, self.window)
+        return KVNeed.keys_values(self.kv_heads, self.head_dim, self.window, self.value_dim, self.keep_first)
 
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
-        qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
         rot = self.position.rotation(batch)
         table = rot.table if rot is not None else None
         pairing = rot.pairing if rot is not None else "halves"
-        if ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
+        eps = 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps)
+        if self.wide:
+            qkv = ops.linear(x, self.qkv, out_dtype=torch.float32)  # the norms' input is not rounded
+            q = ops.qkv_norm_rope_store(qkv, cache.slots if cache.writes else None, self.q_norm, self.k_norm, eps, table,
+                                        cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, self.value_dim,
+                                        self.rt.dtype, pairing)
+            out = ops.paged_attention(q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
+                                      self.scale, self.window, self.value_dim, self.keep_first, self.exact_weights)
+            return ops.linear(out, self.o, accumulate_into=residual, defer=True)
+        qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
+        if not (self.exact_weights or self.keep_first) and ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
                                         self.heads, self.kv_heads, self.head_dim, pairing):
             # a step of single tokens: norm, rotation, cache store and attention are one kernel
             # ... and, with few rows, the reduction of the key splits and the output projection another
@@ -110,7 +151,7 @@ class GQAttention(Mixer):
         )
         out = ops.paged_attention(
             q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
-            self.scale, self.window,
+            self.scale, self.window, None, self.keep_first, self.exact_weights,
         )
         return ops.linear(out, self.o, accumulate_into=residual, defer=True)
 
@@ -120,14 +161,14 @@ class GQAttention(Mixer):
 
     def flops(self, rows) -> int:
         """The four projections, and both attention products over every (query, visible key) pair: a query
-        at position p sees keys ``max(0, p - window + 1) .. p``."""
+        at position p sees keys ``max(0, p - window + 1) .. p`` and the kept first keys."""
         tokens = sum(n for n, _ in rows)
         pairs = 0
         for n, cached in rows:
             for p in (range(cached, cached + n) if self.window else ()):
-                pairs += min(p + 1, self.window)
+                pairs += min(p + 1, self.window + self.keep_first)
             if not self.window:
                 pairs += n * cached + n * (n + 1) // 2
-        width = self.heads * self.head_dim
-        linear = 2 * tokens * self.hidden * (width + 2 * self.kv_heads * self.head_dim) + 2 * tokens * width * self.hidden
-        return linear + 4 * pairs * width
+        qk, vo = self.heads * self.head_dim, self.heads * self.value_dim
+        linear = 2 * tokens * self.hidden * (qk + self.kv_heads * (self.head_dim + self.value_dim)) + 2 * tokens * vo * self.hidden
+        return linear + 2 * pairs * (qk + vo)

@@ -71,10 +71,12 @@ class CachePlane:
 class KVNeed:
     """What a mixer keeps per token, as a list of planes (keys and values of equal or different
     widths, one latent vector, ...). ``window == 0`` keeps every token, ``window > 0`` only the last
-    ``window`` (older pages may be given back)."""
+    ``window`` (older pages may be given back) and, with ``keep_first > 0``, the sequence's first
+    ``keep_first`` tokens as well (their pages never go back while the request lives)."""
 
     planes: tuple[CachePlane, ...]
     window: int = 0
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [p.name for p in self.planes]
@@ -82,10 +84,13 @@ class KVNeed:
             raise ValueError(f"cache planes need distinct names, got {names}")
 
     @classmethod
-    def keys_values(cls, num_kv_heads: int, head_dim: int, window: int = 0) -> "KVNeed":
-        """Keys ``[page_size, head_dim]`` and values ``[head_dim, page_size]`` per KV head: what the
-        attention kernels read."""
-        return cls((CachePlane("k", num_kv_heads, head_dim), CachePlane("v", num_kv_heads, head_dim, token_minor=True)), window)
+    def keys_values(cls, num_kv_heads: int, head_dim: int, window: int = 0, value_dim: int | None = None,
+                    keep_first: int = 0) -> "KVNeed":
+        """Keys ``[page_size, head_dim]`` and values ``[value_dim, page_size]`` per KV head (``value_dim``
+        defaults to ``head_dim``): what the attention kernels read."""
+        return cls((CachePlane("k", num_kv_heads, head_dim),
+                    CachePlane("v", num_kv_heads, head_dim if value_dim is None else value_dim, token_minor=True)),
+                   window, keep_first if window else 0)
 
     @property
     def elements_per_token(self) -> int:

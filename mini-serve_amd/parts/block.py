@@ -37,3 +37,32 @@ class PreNormBlock(Block):
 
     def parameters_bytes(self) -> int:
         return self.mixer_norm.parameters_bytes() + self.ffn_norm.parameters_bytes()
+
+
+@register("block", "parallel")
+class ParallelBlock(Block):
+    """``h += mixer(norm(h)) + feed_forward(norm(h))``: one norm, both sublayers read its output."""
+
+    def __init__(self, spec: PartSpec, rt, mixer, feed_forward):
+        super().__init__(spec, rt, mixer, feed_forward)
+        n = spec["norm"]
+        self.norm = part_class("norm", n)(n, rt)
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        return part_class("norm", spec["norm"]).tensors(spec["norm"])
+
+    def bind(self, tensors) -> None:
+        self.norm.bind(tensors)
+
+    def forward(self, residual, batch, cache, state, pending=None):
+        x = self.norm.forward(residual, add=pending)
+        first = self.mixer.forward(x, batch, cache, state, residual)
+        second = self.feed_forward.forward(x, residual)
+        if first is not None and second is not None:
+            self.rt.ops.add_pending(residual, first)
+            return second
+        return first if first is not None else second
+
+    def parameters_bytes(self) -> int:
+        return self.norm.parameters_bytes()

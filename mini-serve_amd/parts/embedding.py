@@ -3,7 +3,8 @@
 Embedding: ``h = E[token_ids]`` without scaling (miniserve/model/qwen3.py:211), widened to the
 float32 residual stream. Head: ``logits = x W^T`` without bias, scaling or soft-cap
 (miniserve/model/qwen3.py:152,186,195), returned in float32; a tied head reads the embedding's
-tensor itself, no copy (miniserve/model/weights.py:116-119,135-136)."""
+tensor itself, no copy (miniserve/model/weights.py:116-119,135-136). ``logit_scale`` (optional, no
+counterpart in the reference) multiplies the float32 logits."""
 
 from __future__ import annotations
 
@@ -43,6 +44,7 @@ class LinearHead(Head):
         self.vocab = int(spec["vocab_size"])
         self.width = int(spec["width"])
         self.tied_to = spec.get("tied_to")
+        self.logit_scale = float(spec.get("logit_scale") or 1.0)
         self.weight = None
 
     @classmethod
@@ -59,7 +61,8 @@ class LinearHead(Head):
         self.weight = tensors[self.spec["tensor"]]
 
     def forward(self, x):
-        return self.rt.ops.linear(x, self.weight, out_dtype=torch.float32)
+        logits = self.rt.ops.linear(x, self.weight, out_dtype=torch.float32)
+        return logits if self.logit_scale == 1.0 else self.rt.ops.scale_(logits, self.logit_scale)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

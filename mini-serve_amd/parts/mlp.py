@@ -3,7 +3,11 @@
 both (the reference concatenates them, miniserve/model/fused.py:41,195; here their rows alternate in
 runs of 16 where the width allows, so that a matrix kernel's lane holds gate and up of the same output
 and can finish the activation itself); the activation product is evaluated in float32 and rounded
-once; the down projection adds into the residual stream in its epilogue."""
+once; the down projection adds into the residual stream in its epilogue.
+
+``names`` (optional) maps ``gate`` / ``up`` / ``down`` to the tensors' names behind the prefix (default
+``<x>_proj.weight``); ``limit`` belongs to the activations that bound their inputs (``swiglu_clamped``).
+``none`` is the feed-forward of a layer that has none."""
 
 from __future__ import annotations
 
@@ -13,6 +17,20 @@ from ..config.spec import PartSpec
 from .base import FeedForward, TensorSpec
 from .registry import register
 
+def _names(spec: PartSpec) -> dict[str, str]:
+    p = spec.get("prefix", "")
+    given = spec.get("names") or {}
+    return {k: p + given.get(k, f"{k}_proj.weight") for k in ("gate", "up", "down")}
+
+
+@register("feed_forward", "none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: nothing is added."""
+
+    def forward(self, x, residual):
+        return None
+
+
 @register("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
     def __init__(self, spec: PartSpec, rt):
@@ -21,34 +39,33 @@ class GatedMLP(FeedForward):
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
         self.activation = spec.get("activation", "silu")
+        self.limit = float(spec["limit"]) if spec.get("limit") is not None else None
         if self.activation not in rt.ops.ACTIVATIONS:
             raise NotImplementedError(f"activation {self.activation!r} is not supported, expected one of {sorted(rt.ops.ACTIVATIONS)}")
+        if self.activation in rt.ops.ACTIVATIONS_WITH_LIMIT and not (self.limit is not None and self.limit > 0):
+            raise ValueError(f"activation {self.activation!r} needs a positive limit, got {self.limit!r}")
+        self.names = _names(spec)
         self.gate_up = self.down = None
         self.block = 0  # rows per run of gate / up rows in gate_up (0: all gates, then all ups)
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
-        p = spec.get("prefix", "")
         h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
-        return {
-            p + "gate_proj.weight": TensorSpec((i, h)),
-            p + "up_proj.weight": TensorSpec((i, h)),
-            p + "down_proj.weight": TensorSpec((h, i)),
-        }
+        n = _names(spec)
+        return {n["gate"]: TensorSpec((i, h)), n["up"]: TensorSpec((i, h)), n["down"]: TensorSpec((h, i))}
 
     def bind(self, tensors) -> None:
-        p = self.prefix
-        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
-            raise ValueError(f"{p}gate/up projections are stored in different dtypes")
+            raise ValueError(f"{self.prefix}gate/up projections are stored in different dtypes")
         ops = self.rt.ops
         self.block = ops.GATE_BLOCK if self.inter % ops.GATE_BLOCK == 0 else 0
         self.gate_up = ops.interleave_gate_up(g, u) if self.block else torch.cat((g, u), dim=0).contiguous()
-        self.down = tensors[p + "down_proj.weight"]
+        self.down = tensors[self.names["down"]]
 
     def forward(self, x, residual):
         ops = self.rt.ops
-        m = ops.gated_linear(x, self.gate_up, self.activation, out_dtype=self.rt.dtype, block=self.block)
+        m = ops.gated_linear(x, self.gate_up, self.activation, out_dtype=self.rt.dtype, block=self.block, limit=self.limit)
         return ops.linear(m, self.down, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:

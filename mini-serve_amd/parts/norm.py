@@ -33,3 +33,34 @@ class RMSNorm(Norm):
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
+
+
+@register("norm", "layernorm")
+class LayerNorm(Norm):
+    """``y = (x - mean(x)) / sqrt(var(x) + eps) * w + b``, the variance being the mean of the squared
+    deviations; statistics and scaling in float32. ``bias_tensor`` names the bias (None: no bias)."""
+
+    def __init__(self, spec: PartSpec, rt):
+        super().__init__(spec, rt)
+        self.width = int(spec["width"])
+        self.eps = float(spec["eps"])
+        self.weight = self.bias = None
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        out = {spec["tensor"]: TensorSpec((int(spec["width"]),), init="ones")}
+        if spec.get("bias_tensor"):
+            out[spec["bias_tensor"]] = TensorSpec((int(spec["width"]),), init="uniform")
+        return out
+
+    def bind(self, tensors) -> None:
+        self.weight = tensors[self.spec["tensor"]]
+        self.bias = tensors[self.spec["bias_tensor"]] if self.spec.get("bias_tensor") else None
+
+    def forward(self, x, rows=None, add=None):
+        ops = self.rt.ops
+        ops.add_pending(x, add)  # the kernel takes no pending sum along: the stream is brought up to date first
+        return ops.layernorm(x, self.weight, self.bias, self.eps, self.rt.dtype, rows)
+
+    def parameters_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.weight, self.bias) if t is not None)

@@ -1,11 +1,18 @@
-"""Rotary position encoding, rotate-half pairing (j, j + dim/2) over the first ``dim`` elements of
-each head. Frequencies ``inv_freq[j] = 1 / theta**(2j/dim)`` are computed on the host in float32
+"""Rotary position encoding over the first ``dim`` elements of each head, in pairs (j, j + dim/2)
+(``pairing="halves"``, the default) or (2j, 2j + 1) (``pairing="adjacent"``). Frequencies ``inv_freq[j] = 1 / theta**(2j/dim)`` are computed on the host in float32
 exactly as the reference does (miniserve/model/qwen3.py:97-100) and moved once; the angles
 ``float32(position) * inv_freq[j]`` and their cosines and sines are formed in float32 on the device
 once per step, as a table that every layer with the same frequencies shares (the reference builds
-float32 tables per pass, :105-108)."""
+float32 tables per pass, :105-108).
+
+``scaling`` (optional) slows the long wavelengths down, ``{"kind": "wavelength_bands", "factor", "low", "high",
+"original"}``: with wavelength ``l = 2 pi / f``, a frequency stays where ``l < original / high``, becomes ``f / factor``
+where ``l > original / low``, and in between is the blend ``(1 - s) f / factor + s f`` with
+``s = (original / l - low) / (high - low)``. No counterpart in the reference, which refuses ``rope_scaling``."""
 
 from __future__ import annotations
+
+import math
 
 import torch
 
@@ -22,16 +29,42 @@ class Rotary(PositionEncoding):
         self.theta = float(spec["theta"])
         if self.dim < 2 or self.dim % 2:
             raise ValueError(f"rotary dim {self.dim} must be even")
+        self.pairing = spec.get("pairing", "halves")
+        self.scaling = dict(spec["scaling"]) if spec.get("scaling") else None
         expo = torch.arange(0, self.dim, 2, dtype=torch.int64).to(torch.float32) / self.dim
         self.inv_freq_host = 1.0 / (self.theta**expo)
+        if self.scaling is not None:
+            self.inv_freq_host = scale_frequencies(self.inv_freq_host, self.scaling)
         self.inv_freq = self.inv_freq_host.to(rt.device) if rt is not None else None
+        self._key = ("rotary", self.dim, self.theta, tuple(sorted(self.scaling.items())) if self.scaling else None)
 
     def rotation(self, batch) -> Rotation:
-        key = ("rotary", self.dim, self.theta)
-        table = batch.memo.get(key)
+        table = batch.memo.get(self._key)
         if table is None:
-            table = batch.memo[key] = self.rt.ops.rope_table(batch.positions, self.inv_freq)
-        return Rotation(self.dim, table)
+            table = batch.memo[self._key] = self.rt.ops.rope_table(batch.positions, self.inv_freq)
+        return Rotation(self.dim, table, self.pairing)
+
+
+def scale_frequencies(inv_freq: torch.Tensor, scaling: dict) -> torch.Tensor:
+    """The frequencies after ``scaling`` (see the module's text), evaluated in float64 and rounded to float32 once."""
+    kind = scaling.get("kind", "wavelength_bands")
+    if kind != "wavelength_bands":
+        raise NotImplementedError(f"frequency scaling {kind!r} is not supported, expected 'wavelength_bands'")
+    factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    if not (factor > 0 and high > low >= 0 and original > 0):
+        raise ValueError(f"frequency scaling needs factor > 0, high > low >= 0 and original > 0, got {scaling}")
+    out = []
+    shortest, longest = original / high, (original / low if low > 0 else math.inf)
+    for f in inv_freq.to(torch.float64).tolist():
+        wavelength = 2 * math.pi / f
+        if wavelength < shortest:
+            out.append(f)
+        elif wavelength > longest:
+            out.append(f / factor)
+        else:
+            s = (original / wavelength - low) / (high - low)
+            out.append((1 - s) * f / factor + s * f)
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32)
 
 
 @register("position", "none")

@@ -146,9 +146,13 @@ def test_head_sizes_the_kernels_refuse_are_refused_when_the_model_is_built():
         return PartSpec("gqa_attention", base)
 
     GQAttention(spec(), None)
-    for bad in (24, 8, 272, 100):
-        with pytest.raises(ValueError, match="head_dim"):
+    for ok in (24, 8, 100, 256):  # the generic kernel takes any size up to 256
+        GQAttention(spec(head_dim=ok), None)
+    for bad in (272, 0, 1000):
+        with pytest.raises(ValueError, match="head sizes"):
             GQAttention(spec(head_dim=bad), None)
+    with pytest.raises(ValueError, match="head sizes"):
+        GQAttention(spec(value_dim=300), None)
     with pytest.raises(ValueError, match="no multiple"):
         GQAttention(spec(num_heads=5), None)
     with pytest.raises(ValueError, match="scale"):
