@@ -207,3 +207,13 @@ def forward(cfg: dict, weights: dict, tokens, return_layers: bool = False):
     z = layer_norm(x, weights["final.norm"], weights["final.norm.b"], eps)
     logits = z @ weights["embed"].T * float(cfg["logit_scale"])
     return (logits, np.stack(after)) if return_layers else logits
+
+
+def greedy(cfg: dict, weights: dict, prompt, max_new: int) -> list[int]:
+    """One token per pass over the whole sequence so far, first maximal index."""
+    ids, out = list(prompt), []
+    for _ in range(max_new):
+        nxt = int(np.argmax(forward(cfg, weights, ids)[-1]))
+        out.append(nxt)
+        ids.append(nxt)
+    return out

@@ -23,7 +23,8 @@ class Replay:
              "--max-tokens", str(max_tokens), *extra],
             stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1,
         )
-        self.vocab = json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"]
+        cfg = json.loads((Path(model_dir) / "config.json").read_text())
+        self.vocab = cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"]
         self.step_no = 0
 
     def step(self, entries, end=()):
