@@ -169,3 +169,393 @@ extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off,
   else return MS_UNSUPPORTED;
   return launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same recurrences for rows that bring many tokens, in chunks of REC_CHUNK tokens and three passes, so
+// that the work is matrix products over a chunk and every chunk of every row and head has a block of its own:
+//   1. per chunk: the chunk's own contribution to the state at its end, U = sum_j w_j k_j v_j^T (and u = sum_j
+//      w_j k_j), w_j = exp(B - b_j + i_j - a) with b_j the log forget gates summed from the chunk's start through
+//      j, B = b_last, and a = max_j (B - b_j + i_j) (a = 0 for the constant decay, whose weights cannot grow);
+//   2. per (row, head), chunk after chunk: m' = max(B + m, a), S' = exp(B + m - m') S + exp(a - m') U; the state
+//      *before* each chunk takes U's place in the buffer, m and n before it are kept beside it; the state after
+//      the last chunk goes to the slot;
+//   3. per chunk: with the state S0 (n0, m0) before it, m_t by its own recurrence from m0,
+//      o_t = g_t S0^T q_t + sum_(j <= t) P_tj v_j,  P_tj = (q_t . k_j) exp(b_t - b_j + i_j - m_t),  g_t = exp(b_t + m0 - m_t),
+//      n_t . q_t = g_t n0 . q_t + sum_j P_tj, and the normaliser as above.
+// Every exponent is at most zero by the definition of the maxima. All float32; sums are reassociated against the
+// token-by-token kernel, nothing else differs. Head sizes up to REC_CHUNK_MAX_DIM; larger ones take the other kernel.
+#define REC_CHUNK 64
+#define REC_CHUNK_MAX_DIM 128
+
+struct ChunkArgs {
+  RecurrenceArgs r;
+  float* U;    // [chunks, H, D * E]
+  float* u;    // [chunks, H, D]
+  float* cs;   // [chunks, H, 4]: B, a, m before the chunk
+  int rows;
+};
+
+// The chunk `c` of the step: its row, first token and token count; *base = index of the row's first chunk.
+__device__ __forceinline__ void find_chunk(const int* __restrict__ row_start, int rows, int c, int* row, int* first, int* count,
+                                           int* base) {
+  int b = 0, at = 0;
+  for (; b < rows - 1; ++b) {
+    const int nc = (row_start[b + 1] - row_start[b] + REC_CHUNK - 1) / REC_CHUNK;
+    if (c < at + nc) break;
+    at += nc;
+  }
+  *row = b;
+  *base = at;
+  *first = row_start[b] + (c - at) * REC_CHUNK;
+  const int left = row_start[b + 1] - *first;
+  *count = left < REC_CHUNK ? left : REC_CHUNK;
+}
+
+// Log gates of the chunk's tokens into gi[] (and fg[], if given), and the running sums of the log forget gates into
+// bs[] (thread 0 adds).
+__device__ __forceinline__ void chunk_gates(const RecurrenceArgs& a, int h, int first, int count, float* gi, float* bs,
+                                            float* fg = nullptr) {
+  const int tid = threadIdx.x;
+  if (tid < REC_CHUNK) {
+    float i = 0.f, f = 0.f;
+    if (tid < count) {
+      if (a.mode == MS_REC_EXP_GATES) {
+        const float* xr = a.x + (size_t)(first + tid) * a.ld;
+        i = a.cap * tanhf((xr[a.i_off + h] + rec_bias(a.i_bias, a.bias_is_bf16, h)) / a.cap);
+        f = log_sigmoid(a.cap * tanhf((xr[a.f_off + h] + rec_bias(a.f_bias, a.bias_is_bf16, h)) / a.cap));
+      } else {
+        f = logf(a.decay[h]);
+      }
+    }
+    gi[tid] = i;
+    bs[tid] = f;
+    if (fg != nullptr) fg[tid] = f;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float run = 0.f;
+    for (int j = 0; j < REC_CHUNK; ++j) {
+      run += bs[j];
+      bs[j] = run;
+    }
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void rec_chunk_summary_kernel(ChunkArgs c) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const RecurrenceArgs& a = c.r;
+  const int D = a.D, E = a.E, h = blockIdx.y, tid = threadIdx.x;
+  const int DP = (D + 3) & ~3, EP = (E + 3) & ~3;
+  float* Kw = sm;                    // [REC_CHUNK][DP], keys times their weights
+  float* V = Kw + REC_CHUNK * DP;    // [REC_CHUNK][EP]
+  float* gi = V + REC_CHUNK * EP;    // [REC_CHUNK]
+  float* bs = gi + REC_CHUNK;        // [REC_CHUNK]
+  float* wt = bs + REC_CHUNK;        // [REC_CHUNK]
+  __shared__ float amax;
+  int row, first, count, base;
+  find_chunk(a.row_start, c.rows, blockIdx.x, &row, &first, &count, &base);
+  chunk_gates(a, h, first, count, gi, bs);
+  const float B = bs[count - 1];
+  const bool gates = a.mode == MS_REC_EXP_GATES;
+  if (tid == 0) {
+    float mx = 0.f;
+    if (gates) {
+      mx = -INFINITY;
+      for (int j = 0; j < count; ++j) mx = fmaxf(mx, B - bs[j] + gi[j]);
+    }
+    amax = mx;
+  }
+  __syncthreads();
+  if (tid < REC_CHUNK) wt[tid] = tid < count ? expf(B - bs[tid] + gi[tid] - amax) : 0.f;
+  __syncthreads();
+  for (int i = tid; i < REC_CHUNK * DP; i += 256) {
+    const int j = i / DP, d = i % DP;
+    Kw[i] = (j < count && d < D) ? wt[j] * rec_act(a.x[(size_t)(first + j) * a.ld + a.k_off + h * D + d], a.act) : 0.f;
+  }
+  for (int i = tid; i < REC_CHUNK * EP; i += 256) {
+    const int j = i / EP, e = i % EP;
+    V[i] = (j < count && e < E) ? rec_act(a.x[(size_t)(first + j) * a.ld + a.v_off + h * E + e], a.act) : 0.f;
+  }
+  __syncthreads();
+  // thread: 8 rows d0.. of U by 8 columns e0..
+  const int d0 = (tid / 16) * 8, e0 = (tid % 16) * 8;
+  float acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[i][k] = 0.f;
+  if (d0 < DP && e0 < EP) {
+    for (int j = 0; j < count; ++j) {
+      float kd[8], ve[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) kd[i] = d0 + i < DP ? Kw[j * DP + d0 + i] : 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) ve[k] = e0 + k < EP ? V[j * EP + e0 + k] : 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[i][k] = fmaf(kd[i], ve[k], acc[i][k]);
+    }
+  }
+  float* Uo = c.U + ((size_t)blockIdx.x * a.H + h) * D * E;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (d0 + i < D && e0 + k < E) Uo[(size_t)(d0 + i) * E + e0 + k] = acc[i][k];
+  if (gates && tid < D) {
+    float s = 0.f;
+    for (int j = 0; j < count; ++j) s += Kw[j * DP + tid];
+    c.u[((size_t)blockIdx.x * a.H + h) * D + tid] = s;
+  }
+  if (tid == 0) {
+    float* o = c.cs + ((size_t)blockIdx.x * a.H + h) * 4;
+    o[0] = B;
+    o[1] = amax;
+  }
+}
+
+// Pass 2. grid (rows, H, slices): a block owns every slices-th run of 256 elements of the state.
+__global__ __launch_bounds__(256) void rec_chunk_scan_kernel(ChunkArgs c, int slices) {
+  const RecurrenceArgs& a = c.r;
+  const int b = blockIdx.x, h = blockIdx.y, z = blockIdx.z, tid = threadIdx.x;
+  const int DE = a.D * a.E;
+  int base = 0;
+  for (int r = 0; r < b; ++r) base += (a.row_start[r + 1] - a.row_start[r] + REC_CHUNK - 1) / REC_CHUNK;
+  const int nc = (a.row_start[b + 1] - a.row_start[b] + REC_CHUNK - 1) / REC_CHUNK;
+  const bool fresh = a.starts[b] == 0;
+  const bool gates = a.mode == MS_REC_EXP_GATES;
+  const size_t slot = (size_t)a.state_slots[b];
+  float* Sg = a.S + (slot * a.H + h) * (size_t)DE;
+  constexpr int PER = 8;
+  float S[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int idx = (z + slices * i) * 256 + tid;
+    S[i] = (!fresh && idx < DE) ? Sg[idx] : 0.f;
+  }
+  const bool own_n = gates && z == 0 && tid < a.D;
+  float nv = (own_n && !fresh) ? a.n[(slot * a.H + h) * a.D + tid] : 0.f;
+  float m = (gates && !fresh) ? a.m[slot * a.H + h] : 0.f;
+  for (int k = 0; k < nc; ++k) {
+    const size_t at = (size_t)(base + k) * a.H + h;
+    float* Uc = c.U + at * DE;
+    float* csk = c.cs + at * 4;
+    const float B = csk[0], amax = csk[1];
+    float alpha, beta;
+    if (gates) {
+      const float m_new = fmaxf(B + m, amax);
+      alpha = expf(B + m - m_new);
+      beta = expf(amax - m_new);
+      if (z == 0 && tid == 0) csk[2] = m;
+      m = m_new;
+    } else {
+      alpha = expf(B);
+      beta = 1.f;
+    }
+    float t[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = (z + slices * i) * 256 + tid;
+      t[i] = idx < DE ? Uc[idx] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = (z + slices * i) * 256 + tid;
+      if (idx < DE) Uc[idx] = S[i];
+      S[i] = alpha * S[i] + beta * t[i];
+    }
+    if (own_n) {
+      float* uc = c.u + at * a.D;
+      const float t2 = uc[tid];
+      uc[tid] = nv;
+      nv = alpha * nv + beta * t2;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int idx = (z + slices * i) * 256 + tid;
+    if (idx < DE) Sg[idx] = S[i];
+  }
+  if (own_n) a.n[(slot * a.H + h) * a.D + tid] = nv;
+  if (gates && z == 0 && tid == 0) a.m[slot * a.H + h] = m;
+}
+
+__global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const RecurrenceArgs& a = c.r;
+  const int D = a.D, E = a.E, h = blockIdx.y, tid = threadIdx.x;
+  const int DQ = D | 1;              // odd row stride: rows of Q fall into different banks
+  const int EP = (E + 3) & ~3;
+  constexpr int CP = REC_CHUNK + 1;
+  float* V = sm;                     // [REC_CHUNK][EP], first: it is read four floats at a time
+  float* Q = V + REC_CHUNK * EP;     // [REC_CHUNK][DQ]
+  float* Kt = Q + REC_CHUNK * DQ;    // [D][CP], keys transposed
+  float* P = Kt + D * CP;            // [REC_CHUNK][CP]
+  float* gi = P + REC_CHUNK * CP;    // [REC_CHUNK]
+  float* bs = gi + REC_CHUNK;
+  float* mt = bs + REC_CHUNK;
+  float* nq = mt + REC_CHUNK;
+  float* fg = nq + REC_CHUNK;
+  float* n0 = fg + REC_CHUNK;        // [D]
+  int row, first, count, base;
+  find_chunk(a.row_start, c.rows, blockIdx.x, &row, &first, &count, &base);
+  chunk_gates(a, h, first, count, gi, bs, fg);
+  const bool gates = a.mode == MS_REC_EXP_GATES;
+  const size_t at = (size_t)blockIdx.x * a.H + h;
+  const float m0 = gates ? c.cs[at * 4 + 2] : 0.f;
+  if (tid == 0) {
+    float m = m0;  // the running maximum by its own recurrence, as the token-by-token kernel forms it
+    for (int j = 0; j < REC_CHUNK; ++j) {
+      if (gates && j < count) m = fmaxf(fg[j] + m, gi[j]);
+      mt[j] = m;
+    }
+  }
+  for (int i = tid; i < REC_CHUNK * D; i += 256) {
+    const int j = i / D, d = i % D;
+    const bool in = j < count;
+    const float* xr = a.x + (size_t)(first + (in ? j : 0)) * a.ld;
+    Q[j * DQ + d] = in ? rec_act(xr[a.q_off + h * D + d], a.act) * a.q_scale : 0.f;
+    Kt[d * CP + j] = in ? rec_act(xr[a.k_off + h * D + d], a.act) : 0.f;
+  }
+  for (int i = tid; i < REC_CHUNK * EP; i += 256) {
+    const int j = i / EP, e = i % EP;
+    V[i] = (j < count && e < E) ? rec_act(a.x[(size_t)(first + j) * a.ld + a.v_off + h * E + e], a.act) : 0.f;
+  }
+  if (gates && tid < D) n0[tid] = c.u[at * D + tid];
+  __syncthreads();
+  {
+    // scores: thread = 4 tokens t0.. by 4 keys j0..
+    const int t0 = (tid / 16) * 4, j0 = (tid % 16) * 4;
+    float s[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) s[i][k] = 0.f;
+    if (j0 <= t0 + 3) {  // blocks wholly above the diagonal stay zero
+      for (int d = 0; d < D; ++d) {
+        float qv[4], kv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qv[i] = Q[(t0 + i) * DQ + d];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) kv[k] = Kt[d * CP + j0 + k];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int k = 0; k < 4; ++k) s[i][k] = fmaf(qv[i], kv[k], s[i][k]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int t = t0 + i, j = j0 + k;
+        P[t * CP + j] = (j <= t && t < count) ? s[i][k] * expf(bs[t] - bs[j] + gi[j] - mt[t]) : 0.f;
+      }
+  }
+  __syncthreads();
+  if (gates && tid < REC_CHUNK) {
+    float sum = 0.f;
+    for (int j = 0; j <= tid; ++j) sum += P[tid * CP + j];
+    float dot = 0.f;
+    for (int d = 0; d < D; ++d) dot = fmaf(n0[d], Q[tid * DQ + d], dot);
+    nq[tid] = expf(bs[tid] + m0 - mt[tid]) * dot + sum;
+  }
+  // outputs: thread = 8 tokens t0.. by 4 columns e0..
+  const int t0 = (tid / 32) * 8, e0 = (tid % 32) * 4;
+  float o[8][4], in[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[i][k] = in[i][k] = 0.f;
+  if (e0 < EP) {
+    const float* S0 = c.U + at * (size_t)D * E;
+    const bool vec = (E % 4) == 0;
+    for (int d = 0; d < D; ++d) {
+      float sv[4];
+      if (vec) {
+        const float4 v4 = *reinterpret_cast<const float4*>(S0 + (size_t)d * E + e0);
+        sv[0] = v4.x; sv[1] = v4.y; sv[2] = v4.z; sv[3] = v4.w;
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) sv[k] = e0 + k < E ? S0[(size_t)d * E + e0 + k] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float qv = Q[(t0 + i) * DQ + d];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) in[i][k] = fmaf(qv, sv[k], in[i][k]);
+      }
+    }
+    const int jend = t0 + 8 < count ? t0 + 8 : count;
+    for (int j = 0; j < jend; ++j) {
+      const float4 v4 = *reinterpret_cast<const float4*>(V + j * EP + e0);
+      const float vv[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float p = P[(t0 + i) * CP + j];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[i][k] = fmaf(p, vv[k], o[i][k]);
+      }
+    }
+  }
+  __syncthreads();  // nq is complete
+  if (e0 < EP) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int t = t0 + i;
+      if (t >= count) continue;
+      const float g = expf(bs[t] + m0 - mt[t]);
+      const float den = gates ? fmaxf(fabsf(nq[t]), expf(-mt[t])) + 1e-6f : 1.f;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (e0 + k < E) a.out[(size_t)(first + t) * (a.H * E) + h * E + e0 + k] = (g * in[i][k] + o[i][k]) / den;
+    }
+  }
+}
+
+static size_t summary_lds(int D, int E) { return sizeof(float) * ((size_t)REC_CHUNK * (((D + 3) & ~3) + ((E + 3) & ~3)) + 3 * REC_CHUNK); }
+static size_t output_lds(int D, int E) {
+  return sizeof(float) * ((size_t)REC_CHUNK * (D | 1) + (size_t)D * (REC_CHUNK + 1) + (size_t)REC_CHUNK * ((E + 3) & ~3) +
+                          (size_t)REC_CHUNK * (REC_CHUNK + 1) + 5 * REC_CHUNK + D);
+}
+
+// Floats of scratch per chunk and head that ms_gated_recurrence_chunked needs for U; u takes D and cs 4 per chunk and head.
+extern "C" int ms_gated_recurrence_chunk_tokens() { return REC_CHUNK; }
+extern "C" int ms_gated_recurrence_chunk_max_dim() { return REC_CHUNK_MAX_DIM; }
+
+// As ms_gated_recurrence, in chunks. `chunks` = sum over the rows of ceil(tokens / REC_CHUNK) (the host knows the rows'
+// lengths); U [chunks, H, D * E], u [chunks, H, D], cs [chunks, H, 4] are scratch.
+extern "C" int ms_gated_recurrence_chunked(const float* x, int ld, int q_off, int k_off, int v_off, int i_off, int f_off, int H, int D,
+                                           int E, int act, int mode, float q_scale, float cap, const float* decay,
+                                           const void* i_bias, const void* f_bias, int bias_is_bf16, float* S, float* n, float* m,
+                                           const int* row_start, const int* starts, const int* state_slots, float* out, int rows,
+                                           int chunks, float* U, float* u, float* cs, hipStream_t st) {
+  if (rows <= 0 || chunks <= 0) return MS_OK;
+  if (H <= 0 || D <= 0 || E <= 0 || x == nullptr || S == nullptr || out == nullptr || row_start == nullptr || starts == nullptr ||
+      state_slots == nullptr || U == nullptr || cs == nullptr || (act != 0 && act != 1) || q_off < 0 || k_off < 0 || v_off < 0 ||
+      q_off + H * D > ld || k_off + H * D > ld || v_off + H * E > ld)
+    return MS_BAD_ARG;
+  if (mode == MS_REC_DECAY) {
+    if (decay == nullptr) return MS_BAD_ARG;
+  } else if (mode == MS_REC_EXP_GATES) {
+    if (n == nullptr || m == nullptr || u == nullptr || !(cap > 0.f) || i_off < 0 || f_off < 0 || i_off + H > ld || f_off + H > ld)
+      return MS_BAD_ARG;
+  } else {
+    return MS_BAD_ARG;
+  }
+  if (D > REC_CHUNK_MAX_DIM || E > REC_CHUNK_MAX_DIM || H > 65535 || rows > 65535) return MS_UNSUPPORTED;
+  ChunkArgs c{{x, ld, q_off, k_off, v_off, i_off, f_off, H, D, E, act, mode, q_scale, cap, decay, i_bias, f_bias, bias_is_bf16, S, n,
+               m, row_start, starts, state_slots, out},
+              U, u, cs, rows};
+  const size_t lds1 = summary_lds(D, E), lds3 = output_lds(D, E);
+  if (hipFuncSetAttribute((const void*)rec_chunk_summary_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1) != hipSuccess ||
+      hipFuncSetAttribute((const void*)rec_chunk_output_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds3) != hipSuccess)
+    return MS_LAUNCH_FAILED;
+  rec_chunk_summary_kernel<<<dim3(chunks, H), 256, lds1, st>>>(c);
+  const int slices = (D * E + 256 * 8 - 1) / (256 * 8);
+  rec_chunk_scan_kernel<<<dim3(rows, H, slices), 256, 0, st>>>(c, slices);
+  rec_chunk_output_kernel<<<dim3(chunks, H), 256, lds3, st>>>(c);
+  return launch_status();
+}

@@ -35,6 +35,11 @@ _SIGNATURES = {
     "ms_gated_recurrence": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                             _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                             _c_int, _c_void],
+    "ms_gated_recurrence_chunked": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                    _c_float, _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                    _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void],
+    "ms_gated_recurrence_chunk_tokens": [],
+    "ms_gated_recurrence_chunk_max_dim": [],
     "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
     "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
@@ -50,7 +55,10 @@ _SIGNATURES = {
     "ms_gemm_bf16_small_tile_cols": [_c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
-                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
+                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_void],
+    "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
+                                 _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
+    "ms_paged_attention_tiled_tokens": [_c_int, _c_int, _c_int],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void,
@@ -658,10 +666,22 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     fast = (qkv.dtype == BF16 and page == 16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 16
             and qkv.shape[1] % 8 == 0 and dv == head_dim and not (window and keep_first) and not exact_weights)
     if not fast:
-        _check(lib.ms_paged_attention_generic(
-            qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common, None,
-            *meta, t, num_heads, num_kv_heads, head_dim, dv, page, float(scale), int(window), int(keep_first), _stream()),
-            "paged_attention")
+        generic = (qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common)
+        shape = (num_heads, num_kv_heads, head_dim, dv, page, float(scale), int(window), int(keep_first))
+        tile_tokens = lib.ms_paged_attention_tiled_tokens(num_heads // num_kv_heads, head_dim, dv)
+        lens = getattr(batch, "row_lens", None)
+        if not (exact_weights or keep_first or dv != head_dim) or not tile_tokens or lens is None:
+            # the form whose sums have one order whatever the step looks like: float32 results stay bitwise equal
+            _check(lib.ms_paged_attention_generic(*generic, None, *meta, t, *shape, 1, _stream()), "paged_attention")
+            return out
+        # rows that bring one token: eight waves share a head's keys; rows that bring several: tiles of tokens in LDS
+        if n_dec:
+            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, 8, _stream()),
+                   "paged_attention")
+        if n_dec < t:
+            first, count, tiles = _tiles_of(batch, tile_tokens, qkv.device)
+            _check(lib.ms_paged_attention_tiled(*generic, first.data_ptr(), count.data_ptr(), tiles, *meta, *shape, _stream()),
+                   "paged_attention_tiled")
         return out
     if n_dec:
         splits = decode_splits(n_dec, num_kv_heads, batch.max_kv_len)
@@ -700,6 +720,13 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             tiles, rows, *meta, num_heads, num_kv_heads, head_dim, page, float(scale), int(window), _stream()),
             "attention_prefill")
     return out
+
+
+def _tiles_of(batch, tile_tokens: int, device):
+    """``build_prefill_tiles`` of a step, made once per tile size (the step's batch keeps them where it can)."""
+    if hasattr(batch, "prefill_tiles"):
+        return batch.prefill_tiles(tile_tokens)
+    return build_prefill_tiles(batch.row_lens, batch.row_starts_host, tile_tokens, device)
 
 
 def build_prefill_tiles(row_lens, row_starts, tile_tokens: int, device):
@@ -932,6 +959,7 @@ def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_ca
 
 RECURRENCE_MODES = {"decay": 0, "exp_gates": 1}
 RECURRENCE_MAX_DIM = 256
+RECURRENCE_CHUNKED_FROM = 16  # tokens of the longest row from which a step runs the chunked kernels
 
 
 def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
@@ -946,7 +974,12 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     ``mode="decay"``: ``a = decay[head]``, ``b = 1``. ``mode="exp_gates"``: capped exponential gates with a running
     maximum and a normaliser (the kernel's source states the formulas); ``state`` then also holds ``n`` and ``m``.
     ``state["S"]``: float32 ``[slots, heads, dim, value_dim]``; rows with ``starts == 0`` begin from zero.
-    Returns float32 ``[T, heads * value_dim]``."""
+    Returns float32 ``[T, heads * value_dim]``.
+
+    Two kernel families compute the same thing: one walks a row's tokens in order with the state in registers (decode
+    steps, short portions, head sizes above 128); the other works in chunks of 64 tokens (three passes: each chunk's own
+    contribution, a scan over the chunks, each chunk's outputs) and runs when the step's longest row has at least
+    ``RECURRENCE_CHUNKED_FROM`` tokens. They differ by the order of float32 sums only."""
     _dev(x, "x", F32, 2)
     t, ld = x.shape
     if mode not in RECURRENCE_MODES:
@@ -993,7 +1026,22 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
         raise ValueError("one row of x per token of the step is needed")
     out = torch.empty((t, heads * value_dim), dtype=F32, device=x.device)
     bias = i_bias if i_bias is not None else f_bias
-    _check(library().ms_gated_recurrence(
+    lib = library()
+    lens = getattr(batch, "row_lens", None)
+    if lens is not None and max(lens) >= RECURRENCE_CHUNKED_FROM and max(dim, value_dim) <= lib.ms_gated_recurrence_chunk_max_dim():
+        per = lib.ms_gated_recurrence_chunk_tokens()
+        chunks = sum(-(-n // per) for n in lens)
+        U = torch.empty((chunks, heads, dim * value_dim), dtype=F32, device=x.device)
+        u = torch.empty((chunks, heads, dim), dtype=F32, device=x.device) if mode == "exp_gates" else None
+        cs = torch.empty((chunks, heads, 4), dtype=F32, device=x.device)
+        _check(lib.ms_gated_recurrence_chunked(
+            x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], columns.get("i", 0), columns.get("f", 0), heads, dim, value_dim,
+            int(activation == "silu"), RECURRENCE_MODES[mode], float(q_scale), float(cap), _ptr(decay), _ptr(i_bias), _ptr(f_bias),
+            int(bias is not None and bias.dtype == BF16), S.data_ptr(), _ptr(n), _ptr(m), batch.row_start.data_ptr(),
+            batch.starts.data_ptr(), batch.state_slots.data_ptr(), out.data_ptr(), rows, chunks, U.data_ptr(), _ptr(u), cs.data_ptr(),
+            _stream()), "gated_recurrence_chunked")
+        return out
+    _check(lib.ms_gated_recurrence(
         x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], columns.get("i", 0), columns.get("f", 0), heads, dim, value_dim,
         int(activation == "silu"), RECURRENCE_MODES[mode], float(q_scale), float(cap), _ptr(decay), _ptr(i_bias), _ptr(f_bias),
         int(bias is not None and bias.dtype == BF16), S.data_ptr(), _ptr(n), _ptr(m), batch.row_start.data_ptr(),

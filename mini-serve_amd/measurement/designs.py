@@ -1,0 +1,123 @@
+"""Prefill and decode throughput of one architecture beside another of equal size: random weights, layers of the
+sizes real models have, the same step function for both. ``bench.py --design kakunex`` prints what this returns.
+
+A *shape* fixes what the two share: width, query and key/value heads of 128 elements, feed-forward width, window,
+layers, vocabulary. The Kakunex model of a shape repeats (parallel, parallel, parallel, mlstm): window attention that
+keeps the first 4 keys beside a decaying linear attention, and a matrix-memory layer in every fourth place, each
+recurrent mixer with as many heads of 128 x 128 as the attention has query heads. The Qwen3 model of the same
+shape attends within the same window in every layer."""
+
+from __future__ import annotations
+
+import statistics
+import time
+
+SHAPES = {
+    # name: width, heads, kv_heads, feed-forward, window, layers, vocabulary
+    "w1024": dict(width=1024, heads=8, kv_heads=4, ff=3072, window=1024, layers=8, vocab=32768),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, ff=8192, window=2048, layers=8, vocab=32768),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, ff=12288, window=2048, layers=4, vocab=32768),
+}
+HEAD = 128
+KEEP_FIRST = 4
+
+
+def kakunex_config(s: dict) -> dict:
+    decays = [1.0 - 2.0 ** -(3 + 7 * i / max(1, s["heads"] - 1)) for i in range(s["heads"])]
+    left = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": HEAD, "vdim": HEAD, "scale": HEAD ** -0.5,
+            "rot": {"base": 1e6, "dims": HEAD // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+            "mask": {"size": s["window"], "keep_first": KEEP_FIRST}}
+    right = {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "decay": decays}
+    mlp = {"kind": "dense", "ff": s["ff"], "limit": 7.0}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 4 == 3:
+            layers.append({"type": "mlstm", "mixer": {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "gate_cap": 15.0}, "mlp": mlp})
+        else:
+            layers.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp})
+    return {"architecture": "Kakunex", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": layers}
+
+
+def qwen3_config(s: dict) -> dict:
+    return {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_act": "silu", "num_hidden_layers": s["layers"],
+            "hidden_size": s["width"], "num_attention_heads": s["heads"], "num_key_value_heads": s["kv_heads"], "head_dim": HEAD,
+            "intermediate_size": s["ff"], "vocab_size": s["vocab"], "rope_theta": 1e6, "rms_norm_eps": 1e-6,
+            "tie_word_embeddings": True, "max_position_embeddings": 40960, "sliding_window": s["window"],
+            "layer_types": ["sliding_attention"] * s["layers"]}
+
+
+DESIGNS = {"kakunex": kakunex_config, "qwen3": qwen3_config}
+
+
+def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: int, steps: int, warmup: int, say=lambda m: None) -> dict:
+    """Tokens per second of one ``prefill_tokens``-token prompt in one step (median of three after one untimed), and of
+    ``steps`` decode steps of ``batch`` requests that each hold ``context`` tokens (replayed as captured graphs, after
+    ``warmup`` untimed steps)."""
+    import torch
+
+    from ..engine.batch import StepRow
+    from ..engine.runner import ModelRunner
+    from ..loading import random_model
+    from .markers import measured_region
+
+    model = random_model(config, seed=0, dtype=dtype)
+    vocab = model.vocab_size
+    gen = torch.Generator().manual_seed(0)
+
+    def ids(n):
+        return torch.randint(0, vocab, (n,), generator=gen).tolist()
+
+    runner = ModelRunner(model, kv_pool_tokens=max(2 * prefill_tokens, batch * (context + 64)) + 64, max_running=batch,
+                         decode_graph=True)
+    times = []
+    for i in range(4):
+        rc = runner.acquire()
+        toks = ids(prefill_tokens)
+        torch.cuda.synchronize()
+        with measured_region("prefill" if i else "prefill (untimed)"):
+            t0 = time.perf_counter()
+            runner.step([StepRow(rc, toks, [prefill_tokens - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        runner.release(rc)
+    prefill_s = statistics.median(times[1:])
+    say(f"  prefill of {prefill_tokens} tokens: {prefill_s * 1e3:.2f} ms")
+    handles = [runner.acquire() for _ in range(batch)]
+    first = context - warmup - steps
+    for rc in handles:
+        for at in range(0, first, 2048):
+            runner.step([StepRow(rc, ids(min(2048, first - at)), [])])
+    for _ in range(warmup):
+        runner.step([StepRow(rc, ids(1), [0]) for rc in handles])
+    torch.cuda.synchronize()
+    with measured_region("decode"):
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            runner.step([StepRow(rc, ids(1), [0]) for rc in handles])
+        torch.cuda.synchronize()
+        decode_s = (time.perf_counter() - t0) / steps
+    say(f"  decode step of {batch} rows at context {context}: {decode_s * 1e3:.3f} ms")
+    for rc in handles:
+        runner.release(rc)
+    out = {"prefill_tok_s": round(prefill_tokens / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3),
+           "prefill_tflops": round(model.step_flops([(prefill_tokens, 0)]) / prefill_s / 1e12, 1),
+           "decode_tok_s": round(batch / decode_s, 1), "decode_ms_per_step": round(decode_s * 1e3, 4),
+           "decode_weight_gbs": round(model.decode_read_bytes() / decode_s / 1e9, 1),
+           "weights_gb": round(model.decode_read_bytes() / 1e9, 3)}
+    del runner, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def compare(design: str, shapes=None, dtype: str = "bfloat16", prefill_tokens: int = 2048, batch: int = 8, context: int = 2048,
+            steps: int = 32, warmup: int = 8, beside: str = "qwen3", say=lambda m: None) -> dict:
+    """``{shape: {design: figures, beside: figures}}`` for the named shapes (all by default)."""
+    out = {}
+    for name in shapes or sorted(SHAPES):
+        s = SHAPES[name]
+        out[name] = {"shape": dict(s, head=HEAD, keep_first=KEEP_FIRST)}
+        for which in (design, beside):
+            say(f"{name}: {which}")
+            out[name][which] = measure(DESIGNS[which](s), dtype, prefill_tokens, batch, context, steps, warmup, say)
+    return out
