@@ -91,18 +91,41 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] *= corr;
     const int je = j0 + WAVE - 1 < p ? j0 + WAVE - 1 : p;
-    for (int jj = j0; jj <= je; ++jj) {
-      if (jj >= kept && jj < lo) {  // the gap inside a tile that holds kept keys or the window's first keys
-        jj = lo - 1;
-        continue;
-      }
-      const int page = table[jj / page_size];
-      const T* vp = vc + ((size_t)page * Hkv + kvh) * Dv * page_size + (jj % page_size);
-      const float w = ps[wave][jj - j0];
+    if (page_size % VN == 0 && WAVE % page_size == 0) {
+      // Page by page: a lane fetches the page's tokens of its element as 16-byte runs (the page keeps the tokens of
+      // one element side by side). Keys that are not visible carry the weight 0, and fmaf(0, v, o) is o: the sum is
+      // the one over the visible keys in ascending order. Pages that were given back are not read.
+      for (int jp = j0; jp <= je; jp += page_size) {
+        if (jp + page_size <= lo && jp >= kept) continue;  // wholly in the gap
+        const int page = table[jp / page_size];
+        if (page < 0) continue;
+        const T* vp = vc + ((size_t)page * Hkv + kvh) * Dv * page_size;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int e = lane + i * WAVE;
-        if (e < Dv) o[i] = fmaf(w, to_f32(vp[(size_t)e * page_size]), o[i]);
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e >= Dv) continue;
+          for (int u0 = 0; u0 < page_size; u0 += VN) {
+            alignas(16) T vv[VN];
+            *reinterpret_cast<uint4*>(vv) = *reinterpret_cast<const uint4*>(vp + (size_t)e * page_size + u0);
+#pragma unroll
+            for (int u = 0; u < VN; ++u) o[i] = fmaf(ps[wave][jp - j0 + u0 + u], to_f32(vv[u]), o[i]);
+          }
+        }
+      }
+    } else {
+      for (int jj = j0; jj <= je; ++jj) {
+        if (jj >= kept && jj < lo) {  // the gap inside a tile that holds kept keys or the window's first keys
+          jj = lo - 1;
+          continue;
+        }
+        const int page = table[jj / page_size];
+        const T* vp = vc + ((size_t)page * Hkv + kvh) * Dv * page_size + (jj % page_size);
+        const float w = ps[wave][jj - j0];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e < Dv) o[i] = fmaf(w, to_f32(vp[(size_t)e * page_size]), o[i]);
+        }
       }
     }
   }
@@ -230,19 +253,71 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_kernel(
   for (int ti = 0; ti < tiles; ++ti) {
     const int j0 = (ti < kept_tiles ? ti : first_window_tile + (ti - kept_tiles)) * WAVE;
     __syncthreads();  // the tile before has been read
-    for (int i = tid; i < WAVE * D; i += 256) {
-      const int jj = i / D, d = i % D, j = j0 + jj;
-      float v = 0.f;
-      if (j <= p_last && (j >= lo_first || j < kept))
-        v = to_f32(kc[(((size_t)table[j / page_size] * Hkv + kvh) * page_size + (j % page_size)) * D + d]);
-      Kt[d * CP + jj] = v;
-    }
-    for (int i = tid; i < WAVE * Dv; i += 256) {
-      const int e = i / WAVE, jj = i % WAVE, j = j0 + jj;
-      float v = 0.f;
-      if (j <= p_last && (j >= lo_first || j < kept))
-        v = to_f32(vc[(((size_t)table[j / page_size] * Hkv + kvh) * Dv + e) * page_size + (j % page_size)]);
-      Vt[e * CP + jj] = v;
+    constexpr int VN = Vec16<T>::N;
+    if (D % VN == 0 && page_size % VN == 0 && WAVE % page_size == 0) {
+      // 16 bytes a load, all of a thread's loads issued before the first is used: a key's run of VN elements, and a
+      // page's run of VN tokens of one value element.
+      const int kruns = D / VN, vruns = page_size / VN;
+      for (int i0 = 0; i0 < WAVE * kruns; i0 += 4 * 256) {
+        uint4 got[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 256 + tid, jj = i / kruns, d = (i % kruns) * VN, j = j0 + jj;
+          got[u] = make_uint4(0, 0, 0, 0);
+          if (i < WAVE * kruns && j <= p_last && (j >= lo_first || j < kept))
+            got[u] = *reinterpret_cast<const uint4*>(kc + (((size_t)table[j / page_size] * Hkv + kvh) * page_size + (j % page_size)) * D + d);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 256 + tid, jj = i / kruns, d = (i % kruns) * VN;
+          if (i >= WAVE * kruns) continue;
+          alignas(16) T kv[VN];
+          *reinterpret_cast<uint4*>(kv) = got[u];
+#pragma unroll
+          for (int w = 0; w < VN; ++w) Kt[(d + w) * CP + jj] = to_f32(kv[w]);
+        }
+      }
+      const int per_page = Dv * vruns, total = (WAVE / page_size) * per_page;
+      for (int i0 = 0; i0 < total; i0 += 4 * 256) {
+        uint4 got[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 256 + tid, pg = i / per_page, e = (i % per_page) / vruns, part = i % vruns;
+          const int jp = j0 + pg * page_size;  // the page's first key
+          got[u] = make_uint4(0, 0, 0, 0);
+          if (i < total && jp <= p_last && (jp + page_size > lo_first || jp < kept)) {
+            const int page = table[jp / page_size];
+            if (page >= 0) got[u] = *reinterpret_cast<const uint4*>(vc + (((size_t)page * Hkv + kvh) * Dv + e) * page_size + part * VN);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 256 + tid, pg = i / per_page, e = (i % per_page) / vruns, part = i % vruns;
+          if (i >= total) continue;
+          alignas(16) T vv[VN];
+          *reinterpret_cast<uint4*>(vv) = got[u];
+#pragma unroll
+          for (int w = 0; w < VN; ++w) {
+            const int jj = pg * page_size + part * VN + w, j = j0 + jj;
+            Vt[e * CP + jj] = (j <= p_last && (j >= lo_first || j < kept)) ? to_f32(vv[w]) : 0.f;
+          }
+        }
+      }
+    } else {
+      for (int i = tid; i < WAVE * D; i += 256) {
+        const int jj = i / D, d = i % D, j = j0 + jj;
+        float v = 0.f;
+        if (j <= p_last && (j >= lo_first || j < kept))
+          v = to_f32(kc[(((size_t)table[j / page_size] * Hkv + kvh) * page_size + (j % page_size)) * D + d]);
+        Kt[d * CP + jj] = v;
+      }
+      for (int i = tid; i < WAVE * Dv; i += 256) {
+        const int e = i / WAVE, jj = i % WAVE, j = j0 + jj;
+        float v = 0.f;
+        if (j <= p_last && (j >= lo_first || j < kept))
+          v = to_f32(vc[(((size_t)table[j / page_size] * Hkv + kvh) * Dv + e) * page_size + (j % page_size)]);
+        Vt[e * CP + jj] = v;
+      }
     }
     __syncthreads();
     float s[4][4];

@@ -862,10 +862,10 @@ def test_attention_one_token_returns_its_value(ops):
 
 
 def test_attention_refuses_unsupported_head_size(ops):
-    q = rand((1, 3 * 24), F32, 23)
-    kc, vc = rand((1, 1, 16, 24), F32, 24), rand((1, 1, 24, 16), F32, 24)
-    with pytest.raises(ValueError, match="head_dim 24"):
-        ops.paged_attention(q, kc, vc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), make_batch([1], [0]), 1, 1, 24, 1.0, 0)
+    q = rand((1, 3 * 272), F32, 23)
+    kc, vc = rand((1, 1, 16, 272), F32, 24), rand((1, 1, 272, 16), F32, 24)
+    with pytest.raises(ValueError, match="head sizes 272"):
+        ops.paged_attention(q, kc, vc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), make_batch([1], [0]), 1, 1, 272, 1.0, 0)
 
 
 # ------------------------------------------------------------------------------------------ sampling
