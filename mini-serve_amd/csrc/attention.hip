@@ -325,6 +325,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_kernel(
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int k = 0; k < 4; ++k) s[i][k] = 0.f;
+#pragma unroll 4
     for (int d = 0; d < D; ++d) {
       float qv[4], kv[4];
 #pragma unroll
@@ -373,6 +374,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_kernel(
       for (int k = 0; k < 4; ++k) o[i][k] *= c;
     }
     const int jn = p_last - j0 + 1 < WAVE ? p_last - j0 + 1 : WAVE;
+#pragma unroll 4
     for (int jj = 0; jj < jn; ++jj) {
       float vv[4];
 #pragma unroll

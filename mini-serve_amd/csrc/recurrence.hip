@@ -13,10 +13,11 @@
 // sequence starts in this step (starts[row] == 0) begins from zero, every other row from its slot; the state after
 // the row's last token is written back.
 //
-// One block of 256 threads per (row, head) walks the row's tokens in order with the state in registers:
-// thread (s, e) holds S[d][e] for d = s, s + NS, ... (NS = 256 / EP slices, EP the power of two that holds E),
+// One block of 256 threads per (row, head, run of EB value columns) walks the row's tokens in order with the state
+// in registers (the columns of S are independent of one another, so few rows still fill the chip):
+// thread (s, e) holds S[d][e] for d = s, s + NS, ... (NS = 256 / EP slices, EP the power of two that holds EB),
 // adds its part of o_t[e], and the slices' parts meet in LDS in ascending s. What an output element is summed
-// from, and in which order, depends on D and E alone: a token's result does not depend on how the sequence was
+// from, and in which order, depends on D alone: a token's result does not depend on how the sequence was
 // cut into steps or batched.
 #include "common.h"
 
@@ -49,13 +50,15 @@ __device__ __forceinline__ float rec_bias(const void* b, int is_bf16, int h) {
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 template <int PM>
-__global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a, int EP) {
+__global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a, int EP, int EB) {
   __shared__ float qs[2][256], ks[2][256];
   __shared__ float red[256];
   __shared__ float wred[2][4];
   const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int D = a.D, E = a.E;
-  const int NS = 256 / EP, e = tid % EP, s = tid / EP;
+  const int NS = 256 / EP, s = tid / EP;
+  const int e = blockIdx.z * EB + tid % EP;  // this thread's column; columns beyond the block's run or beyond E are idle
+  const bool col = tid % EP < EB && e < E;
   const int per = (D + NS - 1) / NS;
   const int t0 = a.row_start[b], t1 = a.row_start[b + 1];
   const bool fresh = a.starts[b] == 0;
@@ -66,7 +69,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
 #pragma unroll
   for (int i = 0; i < PM; ++i) {
     const int d = s + i * NS;
-    S[i] = (!fresh && i < per && d < D && e < E) ? Sg[(size_t)d * E + e] : 0.f;
+    S[i] = (!fresh && i < per && d < D && col) ? Sg[(size_t)d * E + e] : 0.f;
   }
   float nv = 0.f, m = 0.f;
   if (gates && !fresh) {
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
       const float part = wave_sum(nv * qd);
       if (tid % WAVE == 0) wred[buf][tid / WAVE] = part;
     }
-    const float v = e < E ? rec_act(xr[a.v_off + h * E + e], a.act) : 0.f;
+    const float v = col ? rec_act(xr[a.v_off + h * E + e], a.act) : 0.f;
     __syncthreads();
     float acc = 0.f;
 #pragma unroll
@@ -116,11 +119,11 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
       red[tid] = acc;
       __syncthreads();
       if (s == 0) {
-        acc = red[e];
-        for (int j = 1; j < NS; ++j) acc += red[j * EP + e];
+        acc = red[tid];
+        for (int j = 1; j < NS; ++j) acc += red[j * EP + tid];
       }
     }
-    if (s == 0 && e < E) {
+    if (s == 0 && col) {
       if (gates) {
         const float nq = (wred[buf][0] + wred[buf][1]) + (wred[buf][2] + wred[buf][3]);
         acc = acc / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
@@ -131,9 +134,9 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
 #pragma unroll
   for (int i = 0; i < PM; ++i) {
     const int d = s + i * NS;
-    if (i < per && d < D && e < E) Sg[(size_t)d * E + e] = S[i];
+    if (i < per && d < D && col) Sg[(size_t)d * E + e] = S[i];
   }
-  if (gates) {
+  if (gates && blockIdx.z == 0) {  // every run of columns has formed the same n and m
     if (tid < D) a.n[(slot * a.H + h) * D + tid] = nv;
     if (tid == 0) a.m[slot * a.H + h] = m;
   }
@@ -156,16 +159,16 @@ extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off,
     return MS_BAD_ARG;
   }
   if (D > 256 || E > 256 || H > 65535) return MS_UNSUPPORTED;
-  int EP = 32;
-  while (EP < E) EP *= 2;
+  // Runs of 32 value columns, always: the order of an output's sum then depends on D alone.
+  const int EB = E < 32 ? E : 32, EP = 32;
   const int per = (D + 256 / EP - 1) / (256 / EP);
   RecurrenceArgs a{x, ld, q_off, k_off, v_off, i_off, f_off, H, D, E, act, mode, q_scale, cap, decay, i_bias, f_bias, bias_is_bf16,
                    S, n, m, row_start, starts, state_slots, out};
-  const dim3 grid(rows, H);
-  if (per <= 4) gated_recurrence_kernel<4><<<grid, 256, 0, st>>>(a, EP);
-  else if (per <= 16) gated_recurrence_kernel<16><<<grid, 256, 0, st>>>(a, EP);
-  else if (per <= 64) gated_recurrence_kernel<64><<<grid, 256, 0, st>>>(a, EP);
-  else if (per <= 128) gated_recurrence_kernel<128><<<grid, 256, 0, st>>>(a, EP);
+  const dim3 grid(rows, H, (E + EB - 1) / EB);
+  if (per <= 4) gated_recurrence_kernel<4><<<grid, 256, 0, st>>>(a, EP, EB);
+  else if (per <= 16) gated_recurrence_kernel<16><<<grid, 256, 0, st>>>(a, EP, EB);
+  else if (per <= 64) gated_recurrence_kernel<64><<<grid, 256, 0, st>>>(a, EP, EB);
+  else if (per <= 128) gated_recurrence_kernel<128><<<grid, 256, 0, st>>>(a, EP, EB);
   else return MS_UNSUPPORTED;
   return launch_status();
 }
@@ -286,6 +289,7 @@ __global__ __launch_bounds__(256) void rec_chunk_summary_kernel(ChunkArgs c) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) acc[i][k] = 0.f;
   if (d0 < DP && e0 < EP) {
+#pragma unroll 2
     for (int j = 0; j < count; ++j) {
       float kd[8], ve[8];
 #pragma unroll
@@ -434,6 +438,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) s[i][k] = 0.f;
     if (j0 <= t0 + 3) {  // blocks wholly above the diagonal stay zero
+#pragma unroll 4
       for (int d = 0; d < D; ++d) {
         float qv[4], kv[4];
 #pragma unroll
@@ -472,6 +477,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
   if (e0 < EP) {
     const float* S0 = c.U + at * (size_t)D * E;
     const bool vec = (E % 4) == 0;
+#pragma unroll 4
     for (int d = 0; d < D; ++d) {
       float sv[4];
       if (vec) {
@@ -489,6 +495,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
       }
     }
     const int jend = t0 + 8 < count ? t0 + 8 : count;
+#pragma unroll 4
     for (int j = 0; j < jend; ++j) {
       const float4 v4 = *reinterpret_cast<const float4*>(V + j * EP + e0);
       const float vv[4] = {v4.x, v4.y, v4.z, v4.w};

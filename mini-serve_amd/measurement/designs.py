@@ -25,14 +25,14 @@ KEEP_FIRST = 4
 def kakunex_config(s: dict) -> dict:
     decays = [1.0 - 2.0 ** -(3 + 7 * i / max(1, s["heads"] - 1)) for i in range(s["heads"])]
     left = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": HEAD, "vdim": HEAD, "scale": HEAD ** -0.5,
-            "rot": {"base": 1e6, "dims": HEAD // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+            "rot": {"base": 5e5, "dims": HEAD // 2, "scaling": {"factor": 4.0, "low": 1.0, "high": 8.0, "original": 4096}},
             "mask": {"size": s["window"], "keep_first": KEEP_FIRST}}
     right = {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "decay": decays}
     mlp = {"kind": "dense", "ff": s["ff"], "limit": 7.0}
     layers = []
     for i in range(s["layers"]):
         if i % 4 == 3:
-            layers.append({"type": "mlstm", "mixer": {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "gate_cap": 15.0}, "mlp": mlp})
+            layers.append({"type": "mlstm", "mixer": {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "gate_cap": 10.0}, "mlp": mlp})
         else:
             layers.append({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp})
     return {"architecture": "Kakunex", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,

@@ -51,7 +51,7 @@ KAKUNEX = {
                  linear(1, 16, 8, (0.97,)), ff=48, limit=3.0),
     ]), 11, Init(0.12, (0.6, 1.4))),
     "kxB": (model(257, 80, 1e-6, 1.0, [
-        mlstm(5, 12, 20, 15.0, ff=112, limit=0.7),
+        mlstm(5, 12, 20, 12.0, ff=112, limit=0.7),
         mlstm(1, 40, 40, 2.0, ff=None),
         parallel(attention(6, 1, 20, 12, 0.25, {"base": 50.0, "dims": 4}, {"size": 16, "keep_first": 17}),
                  linear(4, 20, 20, (1.0, 0.3, 0.8, 0.99)), ff=None),

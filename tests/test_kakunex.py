@@ -170,7 +170,7 @@ def test_scaled_frequencies_follow_their_bands():
 
     from miniserve_amd.parts.rotary import scale_frequencies
 
-    for dims, base, scaling in ((64, 1e6, {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 1024}),
+    for dims, base, scaling in ((48, 5e5, {"factor": 6.0, "low": 1.0, "high": 5.0, "original": 2048}),
                                 (8, 100.0, {"factor": 4.0, "low": 1.0, "high": 3.0, "original": 64}),
                                 (6, 8.0, {"factor": 2.0, "low": 0.5, "high": 3.0, "original": 16})):
         plain = K.rotary_frequencies(dims, base, None)

@@ -63,7 +63,7 @@ def test_layer_norm(width, out_dtype):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("groups,group", [(1, 192), (4, 48), (6, 32), (3, 5), (1, 700), (2, 300)])
+@pytest.mark.parametrize("groups,group", [(1, 160), (4, 40), (5, 32), (3, 5), (1, 700), (2, 300)])
 def test_gated_group_norm(groups, group, out_dtype):
     rng = np.random.default_rng(groups * 1000 + group)
     n = groups * group
@@ -76,7 +76,7 @@ def test_gated_group_norm(groups, group, out_dtype):
     close(got, K.unit_rms(x.reshape(5, groups, group), 1e-6).reshape(5, n), out_dtype, "bare")
 
 
-@pytest.mark.parametrize("width", [5, 192, 600])
+@pytest.mark.parametrize("width", [5, 176, 600])
 def test_mean_of_normed_streams(width):
     rng = np.random.default_rng(width)
     r, a, b = rng.normal(size=(6, width)), rng.normal(size=(6, width)) * 10, rng.normal(size=(6, width)) * 0.01
@@ -145,7 +145,7 @@ def plain_attention(q, k, v, scale, size, keep, groups):
     (3, 3, 20, 12, 20, "adjacent", 16, 17),  # a head size that is no multiple of 8; more kept keys than a page
     (6, 1, 64, 64, 0, "halves", 33, 0),      # no rotation, a window without kept keys, one key/value head
     (2, 2, 8, 40, 6, "halves", 0, 0),        # every key visible
-    (2, 1, 32, 32, 16, "adjacent", 40, 20),
+    (2, 1, 32, 32, 16, "adjacent", 45, 19),
 ])
 def test_window_attention_with_kept_first_keys(H, G, D, E, rot, pairing, size, keep, dtype):
     """Norm over the whole projection, rotation, cache store and attention against the plain formulas, in one step and
@@ -225,7 +225,7 @@ def plain_recurrence(q, k, v, a, b):
     return out, S
 
 
-@pytest.mark.parametrize("H,D,E", [(6, 32, 32), (3, 8, 16), (1, 48, 20), (2, 128, 128), (5, 12, 200), (2, 200, 8)])
+@pytest.mark.parametrize("H,D,E", [(6, 24, 40), (3, 8, 16), (1, 48, 20), (2, 128, 128), (5, 12, 200), (2, 200, 8)])
 def test_decay_recurrence_far_keys_and_cuts(H, D, E):
     """One token far back carries a large key and value; a head that hardly decays must still answer a late query along
     that key with it, a head that decays fast must have lost it. Rows of a batch start from their own slots, a row
@@ -275,7 +275,7 @@ def test_decay_recurrence_far_keys_and_cuts(H, D, E):
     close(got[30:], want[1:2], torch.float32, "row 1 goes on")
 
 
-@pytest.mark.parametrize("H,D,E,cap", [(4, 48, 48, 15.0), (2, 8, 24, 3.0), (1, 128, 64, 30.0), (3, 20, 130, 1.0)])
+@pytest.mark.parametrize("H,D,E,cap", [(4, 40, 56, 12.0), (2, 8, 24, 3.0), (1, 128, 64, 30.0), (3, 20, 130, 1.0)])
 def test_exponential_gate_recurrence(H, D, E, cap):
     """Gates from far below to far above zero (the cap bounds them), so that the running maximum moves both ways, the
     normaliser's two branches are both taken and a state that started at zero still counts in the maximum. The
