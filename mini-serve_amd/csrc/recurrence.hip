@@ -194,7 +194,7 @@ struct ChunkArgs {
   RecurrenceArgs r;
   float* U;    // [chunks, H, D * E]
   float* u;    // [chunks, H, D]
-  float* cs;   // [chunks, H, 4]: B, a, m before the chunk
+  double* cs;  // [chunks, H, 4]: B, a, m before the chunk (double: B may be in the hundreds where B + m is small)
   int rows;
 };
 
@@ -215,8 +215,9 @@ __device__ __forceinline__ void find_chunk(const int* __restrict__ row_start, in
 }
 
 // Log gates of the chunk's tokens into gi[] (and fg[], if given), and the running sums of the log forget gates into
-// bs[] (thread 0 adds).
-__device__ __forceinline__ void chunk_gates(const RecurrenceArgs& a, int h, int first, int count, float* gi, float* bs,
+// bs[] (thread 0 adds). The sums are kept in double precision: the kernels need their differences, which may be small
+// where the sums are in the hundreds, and in float32 such a difference would carry the sums' rounding.
+__device__ __forceinline__ void chunk_gates(const RecurrenceArgs& a, int h, int first, int count, float* gi, double* bs,
                                             float* fg = nullptr) {
   const int tid = threadIdx.x;
   if (tid < REC_CHUNK) {
@@ -231,12 +232,12 @@ __device__ __forceinline__ void chunk_gates(const RecurrenceArgs& a, int h, int 
       }
     }
     gi[tid] = i;
-    bs[tid] = f;
+    bs[tid] = (double)f;
     if (fg != nullptr) fg[tid] = f;
   }
   __syncthreads();
   if (tid == 0) {
-    float run = 0.f;
+    double run = 0.0;
     for (int j = 0; j < REC_CHUNK; ++j) {
       run += bs[j];
       bs[j] = run;
@@ -253,24 +254,24 @@ __global__ __launch_bounds__(256) void rec_chunk_summary_kernel(ChunkArgs c) {
   float* Kw = sm;                    // [REC_CHUNK][DP], keys times their weights
   float* V = Kw + REC_CHUNK * DP;    // [REC_CHUNK][EP]
   float* gi = V + REC_CHUNK * EP;    // [REC_CHUNK]
-  float* bs = gi + REC_CHUNK;        // [REC_CHUNK]
-  float* wt = bs + REC_CHUNK;        // [REC_CHUNK]
+  float* wt = gi + REC_CHUNK;        // [REC_CHUNK]
+  __shared__ double bs[REC_CHUNK];
   __shared__ float amax;
   int row, first, count, base;
   find_chunk(a.row_start, c.rows, blockIdx.x, &row, &first, &count, &base);
   chunk_gates(a, h, first, count, gi, bs);
-  const float B = bs[count - 1];
+  const double B = bs[count - 1];
   const bool gates = a.mode == MS_REC_EXP_GATES;
   if (tid == 0) {
     float mx = 0.f;
     if (gates) {
       mx = -INFINITY;
-      for (int j = 0; j < count; ++j) mx = fmaxf(mx, B - bs[j] + gi[j]);
+      for (int j = 0; j < count; ++j) mx = fmaxf(mx, (float)(B - bs[j]) + gi[j]);
     }
     amax = mx;
   }
   __syncthreads();
-  if (tid < REC_CHUNK) wt[tid] = tid < count ? expf(B - bs[tid] + gi[tid] - amax) : 0.f;
+  if (tid < REC_CHUNK) wt[tid] = tid < count ? expf((float)(B - bs[tid]) + gi[tid] - amax) : 0.f;
   __syncthreads();
   for (int i = tid; i < REC_CHUNK * DP; i += 256) {
     const int j = i / DP, d = i % DP;
@@ -314,9 +315,9 @@ __global__ __launch_bounds__(256) void rec_chunk_summary_kernel(ChunkArgs c) {
     c.u[((size_t)blockIdx.x * a.H + h) * D + tid] = s;
   }
   if (tid == 0) {
-    float* o = c.cs + ((size_t)blockIdx.x * a.H + h) * 4;
+    double* o = c.cs + ((size_t)blockIdx.x * a.H + h) * 4;
     o[0] = B;
-    o[1] = amax;
+    o[1] = (double)amax;
   }
 }
 
@@ -341,21 +342,21 @@ __global__ __launch_bounds__(256) void rec_chunk_scan_kernel(ChunkArgs c, int sl
   }
   const bool own_n = gates && z == 0 && tid < a.D;
   float nv = (own_n && !fresh) ? a.n[(slot * a.H + h) * a.D + tid] : 0.f;
-  float m = (gates && !fresh) ? a.m[slot * a.H + h] : 0.f;
+  double m = (gates && !fresh) ? (double)a.m[slot * a.H + h] : 0.0;
   for (int k = 0; k < nc; ++k) {
     const size_t at = (size_t)(base + k) * a.H + h;
     float* Uc = c.U + at * DE;
-    float* csk = c.cs + at * 4;
-    const float B = csk[0], amax = csk[1];
+    double* csk = c.cs + at * 4;
+    const double B = csk[0], amax = csk[1];
     float alpha, beta;
     if (gates) {
-      const float m_new = fmaxf(B + m, amax);
-      alpha = expf(B + m - m_new);
-      beta = expf(amax - m_new);
+      const double m_new = fmax(B + m, amax);
+      alpha = expf((float)(B + m - m_new));
+      beta = expf((float)(amax - m_new));
       if (z == 0 && tid == 0) csk[2] = m;
       m = m_new;
     } else {
-      alpha = expf(B);
+      alpha = expf((float)B);
       beta = 1.f;
     }
     float t[PER];
@@ -383,7 +384,7 @@ __global__ __launch_bounds__(256) void rec_chunk_scan_kernel(ChunkArgs c, int sl
     if (idx < DE) Sg[idx] = S[i];
   }
   if (own_n) a.n[(slot * a.H + h) * a.D + tid] = nv;
-  if (gates && z == 0 && tid == 0) a.m[slot * a.H + h] = m;
+  if (gates && z == 0 && tid == 0) a.m[slot * a.H + h] = (float)m;
 }
 
 __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
@@ -398,19 +399,19 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
   float* Kt = Q + REC_CHUNK * DQ;    // [D][CP], keys transposed
   float* P = Kt + D * CP;            // [REC_CHUNK][CP]
   float* gi = P + REC_CHUNK * CP;    // [REC_CHUNK]
-  float* bs = gi + REC_CHUNK;
-  float* mt = bs + REC_CHUNK;
+  float* mt = gi + REC_CHUNK;
   float* nq = mt + REC_CHUNK;
   float* fg = nq + REC_CHUNK;
   float* n0 = fg + REC_CHUNK;        // [D]
+  __shared__ double bs[REC_CHUNK];
   int row, first, count, base;
   find_chunk(a.row_start, c.rows, blockIdx.x, &row, &first, &count, &base);
   chunk_gates(a, h, first, count, gi, bs, fg);
   const bool gates = a.mode == MS_REC_EXP_GATES;
   const size_t at = (size_t)blockIdx.x * a.H + h;
-  const float m0 = gates ? c.cs[at * 4 + 2] : 0.f;
+  const double m0 = gates ? c.cs[at * 4 + 2] : 0.0;
   if (tid == 0) {
-    float m = m0;  // the running maximum by its own recurrence, as the token-by-token kernel forms it
+    float m = (float)m0;  // the running maximum by its own recurrence, as the token-by-token kernel forms it
     for (int j = 0; j < REC_CHUNK; ++j) {
       if (gates && j < count) m = fmaxf(fg[j] + m, gi[j]);
       mt[j] = m;
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int t = t0 + i, j = j0 + k;
-        P[t * CP + j] = (j <= t && t < count) ? s[i][k] * expf(bs[t] - bs[j] + gi[j] - mt[t]) : 0.f;
+        P[t * CP + j] = (j <= t && t < count) ? s[i][k] * expf((float)(bs[t] - bs[j]) + gi[j] - mt[t]) : 0.f;
       }
   }
   __syncthreads();
@@ -465,7 +466,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
     for (int j = 0; j <= tid; ++j) sum += P[tid * CP + j];
     float dot = 0.f;
     for (int d = 0; d < D; ++d) dot = fmaf(n0[d], Q[tid * DQ + d], dot);
-    nq[tid] = expf(bs[tid] + m0 - mt[tid]) * dot + sum;
+    nq[tid] = expf((float)(bs[tid] + m0 - (double)mt[tid])) * dot + sum;
   }
   // outputs: thread = 8 tokens t0.. by 4 columns e0..
   const int t0 = (tid / 32) * 8, e0 = (tid % 32) * 4;
@@ -513,7 +514,7 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
     for (int i = 0; i < 8; ++i) {
       const int t = t0 + i;
       if (t >= count) continue;
-      const float g = expf(bs[t] + m0 - mt[t]);
+      const float g = expf((float)(bs[t] + m0 - (double)mt[t]));
       const float den = gates ? fmaxf(fabsf(nq[t]), expf(-mt[t])) + 1e-6f : 1.f;
 #pragma unroll
       for (int k = 0; k < 4; ++k)
@@ -522,10 +523,10 @@ __global__ __launch_bounds__(256) void rec_chunk_output_kernel(ChunkArgs c) {
   }
 }
 
-static size_t summary_lds(int D, int E) { return sizeof(float) * ((size_t)REC_CHUNK * (((D + 3) & ~3) + ((E + 3) & ~3)) + 3 * REC_CHUNK); }
+static size_t summary_lds(int D, int E) { return sizeof(float) * ((size_t)REC_CHUNK * (((D + 3) & ~3) + ((E + 3) & ~3)) + 2 * REC_CHUNK); }
 static size_t output_lds(int D, int E) {
   return sizeof(float) * ((size_t)REC_CHUNK * (D | 1) + (size_t)D * (REC_CHUNK + 1) + (size_t)REC_CHUNK * ((E + 3) & ~3) +
-                          (size_t)REC_CHUNK * (REC_CHUNK + 1) + 5 * REC_CHUNK + D);
+                          (size_t)REC_CHUNK * (REC_CHUNK + 1) + 4 * REC_CHUNK + D);
 }
 
 // Floats of scratch per chunk and head that ms_gated_recurrence_chunked needs for U; u takes D and cs 4 per chunk and head.
@@ -533,12 +534,12 @@ extern "C" int ms_gated_recurrence_chunk_tokens() { return REC_CHUNK; }
 extern "C" int ms_gated_recurrence_chunk_max_dim() { return REC_CHUNK_MAX_DIM; }
 
 // As ms_gated_recurrence, in chunks. `chunks` = sum over the rows of ceil(tokens / REC_CHUNK) (the host knows the rows'
-// lengths); U [chunks, H, D * E], u [chunks, H, D], cs [chunks, H, 4] are scratch.
+// lengths); U [chunks, H, D * E], u [chunks, H, D] (float) and cs [chunks, H, 4] (double) are scratch.
 extern "C" int ms_gated_recurrence_chunked(const float* x, int ld, int q_off, int k_off, int v_off, int i_off, int f_off, int H, int D,
                                            int E, int act, int mode, float q_scale, float cap, const float* decay,
                                            const void* i_bias, const void* f_bias, int bias_is_bf16, float* S, float* n, float* m,
                                            const int* row_start, const int* starts, const int* state_slots, float* out, int rows,
-                                           int chunks, float* U, float* u, float* cs, hipStream_t st) {
+                                           int chunks, float* U, float* u, double* cs, hipStream_t st) {
   if (rows <= 0 || chunks <= 0) return MS_OK;
   if (H <= 0 || D <= 0 || E <= 0 || x == nullptr || S == nullptr || out == nullptr || row_start == nullptr || starts == nullptr ||
       state_slots == nullptr || U == nullptr || cs == nullptr || (act != 0 && act != 1) || q_off < 0 || k_off < 0 || v_off < 0 ||

@@ -964,7 +964,8 @@ RECURRENCE_CHUNKED_FROM = 16  # tokens of the longest row from which a step runs
 
 def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
                      mode: str, activation: str | None = None, q_scale: float = 1.0, decay: torch.Tensor | None = None,
-                     cap: float = 0.0, i_bias: torch.Tensor | None = None, f_bias: torch.Tensor | None = None) -> torch.Tensor:
+                     cap: float = 0.0, i_bias: torch.Tensor | None = None, f_bias: torch.Tensor | None = None,
+                     chunks: bool = True) -> torch.Tensor:
     """A linear recurrence over a matrix state per (request, head): ``S_t = a_t S_(t-1) + b_t k_t v_t^T``,
     ``o_t = S_t^T q_t``, for the step's rows (``batch.row_start``, ``batch.starts``, ``batch.state_slots``), in float32.
 
@@ -979,7 +980,8 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     Two kernel families compute the same thing: one walks a row's tokens in order with the state in registers (decode
     steps, short portions, head sizes above 128); the other works in chunks of 64 tokens (three passes: each chunk's own
     contribution, a scan over the chunks, each chunk's outputs) and runs when the step's longest row has at least
-    ``RECURRENCE_CHUNKED_FROM`` tokens. They differ by the order of float32 sums only."""
+    ``RECURRENCE_CHUNKED_FROM`` tokens. They differ by the order of float32 sums only. ``chunks=False`` keeps to the
+    first (the chunked kernels take the decays' logarithms: a decay of zero has none)."""
     _dev(x, "x", F32, 2)
     t, ld = x.shape
     if mode not in RECURRENCE_MODES:
@@ -1028,12 +1030,13 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     bias = i_bias if i_bias is not None else f_bias
     lib = library()
     lens = getattr(batch, "row_lens", None)
-    if lens is not None and max(lens) >= RECURRENCE_CHUNKED_FROM and max(dim, value_dim) <= lib.ms_gated_recurrence_chunk_max_dim():
+    if (chunks and lens is not None and max(lens) >= RECURRENCE_CHUNKED_FROM
+            and max(dim, value_dim) <= lib.ms_gated_recurrence_chunk_max_dim()):
         per = lib.ms_gated_recurrence_chunk_tokens()
         chunks = sum(-(-n // per) for n in lens)
         U = torch.empty((chunks, heads, dim * value_dim), dtype=F32, device=x.device)
         u = torch.empty((chunks, heads, dim), dtype=F32, device=x.device) if mode == "exp_gates" else None
-        cs = torch.empty((chunks, heads, 4), dtype=F32, device=x.device)
+        cs = torch.empty((chunks, heads, 4), dtype=torch.float64, device=x.device)
         _check(lib.ms_gated_recurrence_chunked(
             x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], columns.get("i", 0), columns.get("f", 0), heads, dim, value_dim,
             int(activation == "silu"), RECURRENCE_MODES[mode], float(q_scale), float(cap), _ptr(decay), _ptr(i_bias), _ptr(f_bias),

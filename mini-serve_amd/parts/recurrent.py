@@ -90,6 +90,7 @@ class DecayLinearAttention(_RecurrentMixer):
         if not all(0.0 <= d <= 1.0 for d in decay):
             raise ValueError(f"decays must lie in [0, 1], got {decay}")
         self.decay = torch.tensor(decay, dtype=torch.float32, device=rt.device) if rt is not None else None
+        self.chunks = min(decay) > 1e-30  # the chunked kernels work with the decays' logarithms
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -109,7 +110,7 @@ class DecayLinearAttention(_RecurrentMixer):
         ops = self.rt.ops
         x32 = ops.linear(x, self.proj, out_dtype=torch.float32)
         o = ops.gated_recurrence(x32, self.columns, self.heads, self.dim, self.value_dim, batch, state, mode="decay",
-                                 activation="silu", decay=self.decay)
+                                 activation="silu", decay=self.decay, chunks=self.chunks)
         return self._finish(o, x32, self.heads * self.value_dim, residual)
 
 

@@ -225,7 +225,7 @@ def plain_recurrence(q, k, v, a, b):
     return out, S
 
 
-@pytest.mark.parametrize("H,D,E", [(6, 24, 40), (3, 8, 16), (1, 48, 20), (2, 128, 128), (5, 12, 200), (2, 200, 8)])
+@pytest.mark.parametrize("H,D,E", [(6, 24, 40), (3, 8, 16), (1, 48, 20), (2, 128, 128), (5, 12, 200), (2, 200, 8), (2, 7, 10), (3, 33, 1)])
 def test_decay_recurrence_far_keys_and_cuts(H, D, E):
     """One token far back carries a large key and value; a head that hardly decays must still answer a late query along
     that key with it, a head that decays fast must have lost it. Rows of a batch start from their own slots, a row
@@ -275,13 +275,14 @@ def test_decay_recurrence_far_keys_and_cuts(H, D, E):
     close(got[30:], want[1:2], torch.float32, "row 1 goes on")
 
 
-@pytest.mark.parametrize("H,D,E,cap", [(4, 40, 56, 12.0), (2, 8, 24, 3.0), (1, 128, 64, 30.0), (3, 20, 130, 1.0)])
+@pytest.mark.parametrize("H,D,E,cap", [(4, 40, 56, 12.0), (2, 8, 24, 3.0), (1, 128, 64, 30.0), (3, 20, 130, 1.0), (2, 6, 9, 4.0), (2, 1, 127, 6.0)])
 def test_exponential_gate_recurrence(H, D, E, cap):
     """Gates from far below to far above zero (the cap bounds them), so that the running maximum moves both ways, the
     normaliser's two branches are both taken and a state that started at zero still counts in the maximum. The
     running maximum is a float32 sum of gates as large as the cap: what each addition rounds away (the cap times
     2^-24) stays in the state's scale and shows where the normaliser's floor exp(-m) decides, so the bound grows
-    with the cap."""
+    with the cap. And the normaliser n . q is a sum of terms of both signs: where it is small beside them, float32
+    has lost what the sum cancelled, in any order of summation, so a token's bound also grows with that ratio."""
     o = ops()
     rng = np.random.default_rng(E)
     T = 300
@@ -292,6 +293,7 @@ def test_exponential_gate_recurrence(H, D, E, cap):
     x[:40, cols["i"] : cols["i"] + H] = -abs(x[:40, cols["i"] : cols["i"] + H])  # early on the maximum is the zero state's
     bi, bf = rng.normal(size=H), rng.normal(size=H)
     want = np.zeros((T, H * E))
+    lost = np.zeros((T, H * E))  # sum |n_d q_d| over the normaliser, per output element
     branches = set()
     for h in range(H):
         q = x[:, h * D : (h + 1) * D] * D**-0.5
@@ -307,6 +309,7 @@ def test_exponential_gate_recurrence(H, D, E, cap):
             m = m_new
             branches.add(abs(n @ q[t]) > math.exp(-m))
             want[t, h * E : (h + 1) * E] = S.T @ q[t] / (max(abs(n @ q[t]), math.exp(-m)) + 1e-6)
+            lost[t, h * E : (h + 1) * E] = np.abs(n * q[t]).sum() / (max(abs(n @ q[t]), math.exp(-m)) + 1e-6)
     assert branches == {True, False}
     state = {"S": torch.full((3, H, D, E), 3.0, device=DEV), "n": torch.full((3, H, D), -2.0, device=DEV),
              "m": torch.full((3, H), 9.0, device=DEV)}
@@ -320,8 +323,9 @@ def test_exponential_gate_recurrence(H, D, E, cap):
             got.append(o.gated_recurrence(dev(x[at : at + n]), cols, H, D, E, b, state, mode="exp_gates", q_scale=D**-0.5, cap=cap,
                                           i_bias=dev(bi), f_bias=dev(bf)))
             at += n
-        err = np.abs(torch.cat(got).cpu().numpy() - want).max()
-        assert err <= 1e-5 * max(2.0, cap) * np.abs(want).max(), f"cuts {cuts[:3]}: {err:.3e}"
+        err = np.abs(torch.cat(got).cpu().numpy() - want)
+        bound = 1e-5 * max(2.0, cap) * np.abs(want).max() + 5e-7 * lost * np.abs(want)
+        assert (err <= bound).all(), f"cuts {cuts[:3]}: {(err / bound).max():.2f} times the bound"
 
 
 # ---------------------------------------------------------------- whole models
