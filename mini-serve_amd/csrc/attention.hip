@@ -174,7 +174,7 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
                                           hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (D <= 0 || D > MAX_HEAD_DIM || Dv <= 0 || Dv > MAX_HEAD_DIM || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 ||
-      window < 0 || keep_first < 0 || table_width <= 0 || Hq > 65535 || q_stride < Hq * D || (waves != 1 && waves != 8))
+      window < 0 || keep_first < 0 || table_width <= 0 || Hq > 65535 || q_stride < Hq * D || (waves != 1 && waves != 8 && waves != 16))
     return MS_BAD_ARG;
   if (window == 0) keep_first = 0;  // every key is visible anyway
   dim3 grid(tokens, Hq);
@@ -183,9 +183,9 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
                                                                     table_width, token_list, token_row, pos, (T*)out, Hq, Hkv, D, Dv, \
                                                                     page_size, scale, window, keep_first)
   if (is_bf16) {
-    if (waves == 8) GA(bf16, 8); else GA(bf16, 1);
+    if (waves == 16) GA(bf16, 16); else if (waves == 8) GA(bf16, 8); else GA(bf16, 1);
   } else {
-    if (waves == 8) GA(float, 8); else GA(float, 1);
+    if (waves == 16) GA(float, 16); else if (waves == 8) GA(float, 8); else GA(float, 1);
   }
 #undef GA
   return launch_status();

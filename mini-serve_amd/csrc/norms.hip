@@ -10,26 +10,48 @@
 
 // ---------------------------------------------------------------------------------------------
 // y[r, :] = (x[row(r), :] - mean) * rsqrt(var + eps) * w + b, var = mean of squared deviations.
-// One block per row. Mean first, then the deviations' squares: two passes over the row, which stays
-// in the cache between them. Sums per thread in ascending element order, then a fixed block order.
+// One block per row. Mean first, then the deviations' squares: two passes over the row, of which a thread keeps
+// its first eight elements in registers. Sums per thread in ascending element order, then a fixed block order.
 template <typename TW, typename TO, int NT>
 __global__ __launch_bounds__(NT) void layernorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
                                                        const TW* __restrict__ b, TO* __restrict__ y,
                                                        const int* __restrict__ rows, int width, float eps) {
   __shared__ float red[NT / WAVE];
+  constexpr int KEEP = 8;  // elements a thread keeps in registers between the passes (wider rows are read again)
   const int r = blockIdx.x;
   const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
+  float kept[KEEP];
   float s = 0.f;
-  for (int e = threadIdx.x; e < width; e += NT) s += xr[e];
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int e = threadIdx.x + i * NT;
+    kept[i] = e < width ? xr[e] : 0.f;
+    s += kept[i];
+  }
+  for (int e = threadIdx.x + KEEP * NT; e < width; e += NT) s += xr[e];
   const float mean = block_sum<NT>(s, red) / (float)width;
   float v = 0.f;
-  for (int e = threadIdx.x; e < width; e += NT) {
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const float d = kept[i] - mean;
+    if (threadIdx.x + i * NT < width) v += d * d;
+  }
+  for (int e = threadIdx.x + KEEP * NT; e < width; e += NT) {
     const float d = xr[e] - mean;
     v += d * d;
   }
   const float rstd = 1.f / sqrtf(block_sum<NT>(v, red) / (float)width + eps);
   TO* yr = y + (size_t)r * width;
-  for (int e = threadIdx.x; e < width; e += NT) {
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int e = threadIdx.x + i * NT;
+    if (e < width) {
+      float o = (kept[i] - mean) * rstd * to_f32(w[e]);
+      if (b != nullptr) o += to_f32(b[e]);
+      yr[e] = from_f32<TO>(o);
+    }
+  }
+  for (int e = threadIdx.x + KEEP * NT; e < width; e += NT) {
     float o = (xr[e] - mean) * rstd * to_f32(w[e]);
     if (b != nullptr) o += to_f32(b[e]);
     yr[e] = from_f32<TO>(o);

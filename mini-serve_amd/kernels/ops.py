@@ -676,7 +676,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             return out
         # rows that bring one token: eight waves share a head's keys; rows that bring several: tiles of tokens in LDS
         if n_dec:
-            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, 8, _stream()),
+            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES, _stream()),
                    "paged_attention")
         if n_dec < t:
             first, count, tiles = _tiles_of(batch, tile_tokens, qkv.device)
@@ -956,6 +956,8 @@ def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_ca
 
 
 # ------------------------------------------------------------------------------------- linear recurrences
+
+DECODE_GENERIC_WAVES = 16  # waves that share a (token, head) in the float32 attention of single-token rows (8 or 16)
 
 RECURRENCE_MODES = {"decay": 0, "exp_gates": 1}
 RECURRENCE_MAX_DIM = 256

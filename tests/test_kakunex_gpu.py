@@ -146,6 +146,8 @@ def plain_attention(q, k, v, scale, size, keep, groups):
     (6, 1, 64, 64, 0, "halves", 33, 0),      # no rotation, a window without kept keys, one key/value head
     (2, 2, 8, 40, 6, "halves", 0, 0),        # every key visible
     (2, 1, 32, 32, 16, "adjacent", 45, 19),
+    (2, 1, 128, 128, 32, "adjacent", 70, 9),   # the largest head the tiled kernel takes
+    (1, 1, 160, 136, 0, "halves", 50, 3),      # beyond it: the kernel with a wave (or several) per token and head
 ])
 def test_window_attention_with_kept_first_keys(H, G, D, E, rot, pairing, size, keep, dtype):
     """Norm over the whole projection, rotation, cache store and attention against the plain formulas, in one step and
@@ -186,10 +188,10 @@ def test_window_attention_with_kept_first_keys(H, G, D, E, rot, pairing, size, k
     # the test's inputs do what they are for: one key more or fewer in the window or among the kept keys shows
     if size:
         off = plain_attention(q, k, v, scale, size + 1, keep, H // G).reshape(T, H * E)
-        assert np.abs(off - want).max() > 0.15 * np.abs(want).max()
+        assert np.abs(off - want).max() > 0.1 * np.abs(want).max()
     if keep:
         off = plain_attention(q, k, v, scale, size, keep - 1, H // G).reshape(T, H * E)
-        assert np.abs(off - want).max() > 0.15 * np.abs(want).max()
+        assert np.abs(off - want).max() > 0.1 * np.abs(want).max()
 
     pages = -(-T // page)
     for cuts in ([T], [100] + [1] * 50, [2, 3, 64, 5, 2, 31, 1, 1, 40, 1]):
@@ -208,8 +210,9 @@ def test_window_attention_with_kept_first_keys(H, G, D, E, rot, pairing, size, k
             got.append(o.paged_attention(qq, kc, vc, table, b, H, G, D, scale, size, E, keep, True))
             at += n
         got = torch.cat(got)
-        if dtype == torch.float32:
-            close(got, want, dtype, f"cuts {cuts[:3]}")
+        if dtype == torch.float32:  # scores are sums of D float32 products and stand in an exponent: the bound grows with D
+            err = np.abs(got.cpu().numpy() - want).max()
+            assert err <= 2e-5 * max(1.0, D / 64) * np.abs(want).max(), f"cuts {cuts[:3]}: {err:.3e}"
         else:
             err = np.abs(got.float().cpu().numpy() - want)
             assert err.max() <= 0.06 * np.abs(want).max() and np.sqrt((err**2).mean()) <= 0.01 * np.abs(want).max(), f"cuts {cuts[:3]}"
