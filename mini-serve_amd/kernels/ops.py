@@ -674,7 +674,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             # the form whose sums have one order whatever the step looks like: float32 results stay bitwise equal
             _check(lib.ms_paged_attention_generic(*generic, None, *meta, t, *shape, 1, _stream()), "paged_attention")
             return out
-        # rows that bring one token: eight waves share a head's keys; rows that bring several: tiles of tokens in LDS
+        # rows that bring one token: several waves share a head's keys; rows that bring several: tiles of tokens in LDS
         if n_dec:
             _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES, _stream()),
                    "paged_attention")
