@@ -63,6 +63,12 @@ KAKUNEX = {
                  linear(3, 4, 4, (0.6, 0.7, 0.8)), ff=None),
         mlstm(3, 32, 32, 8.0, ff=80, limit=1.5),
     ]), 13, Init(0.1, (0.7, 1.3))),
+    # sizes that are multiples of nothing: width, feed-forward, vocabulary and every head size odd or twice an odd number
+    "kxD": (model(77, 90, 1e-5, 2.5, [
+        parallel(attention(3, 1, 10, 6, 0.4, {"base": 300.0, "dims": 10}, {"size": 21, "keep_first": 3}),
+                 linear(2, 5, 7, (0.85, 0.99)), ff=50, limit=1.2),
+        mlstm(3, 9, 11, 7.0, ff=34, limit=2.0),
+    ]), 14, Init(0.1, (0.6, 1.4))),
 }
 
 
