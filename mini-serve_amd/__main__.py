@@ -181,11 +181,12 @@ def main(argv=None) -> int:
     w.add_argument("rest", nargs=argparse.REMAINDER)
     w.set_defaults(fn=None)
 
-    args = ap.parse_args(argv)
-    if args.command == "random-weights":
+    argv = sys.argv[1:] if argv is None else list(argv)
+    if argv and argv[0] == "random-weights":  # its own parser takes everything behind the command's name
         from .weights.random_init import main as rw_main
 
-        return rw_main(args.rest)
+        return rw_main(argv[1:])
+    args = ap.parse_args(argv)
     return args.fn(args)
 
 

@@ -1,11 +1,13 @@
 """Named ``config.json`` dictionaries: two tiny shapes that differ in every size and option, one
-tiny windowed shape, and the three benchmark shapes (random weights; no checkpoint is fetched).
+tiny windowed shape, the three benchmark shapes, and one tiny Kakunex model (random weights; no checkpoint is fetched).
 
 The reference names models by size and maps them to pinned downloads
 (miniserve/model/weights.py:24-29); without a network the names map to shapes instead.
 """
 
 from __future__ import annotations
+
+import copy
 
 
 def _qwen3(**kw) -> dict:
@@ -61,8 +63,33 @@ PRESETS: dict[str, dict] = {
 }
 
 
+def _kakunex_tiny() -> dict:
+    """Three layers that hold every part of the architecture once: windowed attention that keeps the first keys beside
+    a decaying linear attention, an mLSTM layer without a feed-forward, and an attention that rotates the whole head."""
+    bands = {"factor": 4.0, "low": 1.0, "high": 3.0, "original": 64}
+
+    def pair(heads, kv_heads, dim, vdim, rot, mask, lin_heads, lin_dim, lin_vdim, decay, ff):
+        left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "rot": rot, "mask": mask}
+        right = {"heads": lin_heads, "dim": lin_dim, "vdim": lin_vdim, "decay": decay}
+        return {"type": "parallel", "mixer": {"left": left, "right": right},
+                "mlp": {"kind": "dense", "ff": ff, "limit": 4.0} if ff else None}
+
+    return {
+        "architecture": "Kakunex", "vocab": 311, "width": 96, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
+        "layers": [
+            pair(4, 2, 32, 16, {"base": 1000.0, "dims": 16, "scaling": bands}, {"size": 24, "keep_first": 6}, 3, 16, 32,
+                 [0.7, 0.95, 0.999], 160),
+            {"type": "mlstm", "mixer": {"heads": 2, "dim": 24, "vdim": 48, "gate_cap": 8.0}, "mlp": None},
+            pair(3, 3, 16, 32, {"base": 1000.0, "dims": 16}, {"size": 40, "keep_first": 0}, 2, 8, 48, [0.9, 0.99], 128),
+        ],
+    }
+
+
+PRESETS["kakunex-tiny"] = _kakunex_tiny()
+
+
 def preset(name: str) -> dict:
     try:
-        return dict(PRESETS[name])
+        return copy.deepcopy(PRESETS[name])
     except KeyError:
         raise ValueError(f"unknown preset {name!r}, expected one of {sorted(PRESETS)}") from None

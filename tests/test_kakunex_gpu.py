@@ -498,3 +498,29 @@ def test_trace_replay(folders, plain_logits, tmp_path):
         assert run.close() == 0
     wa, wb = plain_logits(name, a), plain_logits(name, b)
     check_logits(np.concatenate(got), np.stack([wa[0], wa[32], wa[34], wb[20], wa[69], wb[3], wb[20]]), "float32", "trace replay")
+
+
+def test_command_line_random_weights_generate_and_stress(tmp_path):
+    """The command line serves the architecture like any other: a folder of random weights from the named preset,
+    greedy generation from it against the plain implementation, and a sampled load that returns every page and slot."""
+    import json
+    import subprocess
+    import sys
+
+    from replay_util import ROOT
+
+    folder = tmp_path / "m"
+    run = lambda *a: subprocess.run([sys.executable, "-m", "miniserve_amd", *a], capture_output=True, text=True, cwd=str(ROOT), timeout=110)
+    res = run("random-weights", "--preset", "kakunex-tiny", "--seed", "5", "--std", "0.1", "--norm-range", "0.6", "1.4", "--out", str(folder))
+    assert res.returncode == 0, res.stderr[-2000:]
+    cfg, w = read_model_folder(folder)
+    prompt = np.random.default_rng(8).integers(0, cfg["vocab"], size=30).tolist()
+    res = run("generate", "--model", str(folder), "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)),
+              "--max-new-tokens", "8", "--kv-pool-tokens", "256")
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert json.loads(res.stdout.strip().splitlines()[-1])["outputs"] == [K.greedy(cfg, w, prompt, 8)]
+    res = run("stress", "--model", str(folder), "--num-requests", "12", "--prompt-len", "4", "90", "--max-new-tokens", "1", "20",
+              "--kv-pool-tokens", "640", "--max-running", "4", "--chunked-prefill-size", "64", "--temperature", "0.7", "--top-p", "0.9")
+    assert res.returncode == 0, res.stdout[-1000:] + res.stderr[-2000:]
+    report = json.loads(res.stdout.strip().splitlines()[-1])
+    assert report["finished"] == 12 and report["idle"] and report["engine"]["architecture"] == "Kakunex"
