@@ -44,7 +44,7 @@ class LinearHead(Head):
         self.vocab = int(spec["vocab_size"])
         self.width = int(spec["width"])
         self.tied_to = spec.get("tied_to")
-        self.logit_scale = float(spec.get("logit_scale") or 1.0)
+        self.logit_scale = 1.0 if spec.get("logit_scale") is None else float(spec["logit_scale"])
         self.weight = None
 
     @classmethod
