@@ -438,3 +438,201 @@ extern "C" int ms_paged_attention_tiled(const void* q, int q_stride, const void*
   }
   return launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// The tiled form on the matrix cores, for bfloat16 storage with 16-token pages, head sizes that are multiples of 32
+// (keys) and 16 (values) up to 128: the same tiles of tokens and of 64 keys, the same masks, float32 results of the
+// same meaning. Queries and keys are bfloat16 as stored, so their products are exact in float32 and the scores are
+// float32 sums of them (v_mfma_f32_16x16x32_bf16). The softmax weights stay float32: each is cut into three
+// bfloat16 pieces (hi = bf16(p), mid = bf16(p - hi), lo = bf16(p - hi - mid): 24 bits of mantissa, p itself), and the
+// second product runs once per piece into the same float32 accumulators, so what meets the values is the float32
+// weight, not a rounding of it.
+//   A wave owns 16 of the block's 64 query rows. Scores: A = 16 query rows x 32 elements, B = 32 elements x 16 keys,
+//   both one 16-byte load per lane straight from global memory; a lane then holds one key of four rows
+//   (rows 4 (lane / 16) + r), a row's maximum and sum meet over the 16 lanes that share it. The weights go through a
+//   wave's own LDS rows to change hands (the second product wants a row's 8 consecutive keys in one lane); values:
+//   B = 32 keys x 16 elements, 8 consecutive tokens of one element being one 16-byte load from the transposed page.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+#define MFMA_PAGE 16
+
+__device__ __forceinline__ bf16x8 load_bf16x8(const bf16* p) {
+  union { uint4 u; bf16x8 v; } x;
+  x.u = *reinterpret_cast<const uint4*>(p);
+  return x.v;
+}
+__device__ __forceinline__ bf16x8 zero_bf16x8() {
+  union { uint4 u; bf16x8 v; } x;
+  x.u = make_uint4(0, 0, 0, 0);
+  return x.v;
+}
+
+template <int D, int DV>
+__global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
+    const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
+    int Hq, int Hkv, float scale, int window, int keep_first) {
+  constexpr int PS = WAVE + 4;  // floats between a wave's rows of weights
+  __shared__ __attribute__((aligned(16))) float Pw[4][16][PS];
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
+  const int kvh = blockIdx.y, g = Hq / Hkv;
+  const int first = tile_first[blockIdx.x], count = tile_count[blockIdx.x], rows = count * g;
+  const int* table = block_table + (size_t)token_row[first] * table_width;
+  const int p_first = pos[first], p_last = p_first + count - 1;
+  const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  const int kept = keep_first < lo_first ? keep_first : lo_first;
+
+  // this lane's query row as the A operand: row 16 wave + l16, elements 32 kk + 8 grp .. + 7
+  bf16x8 qf[D / 32];
+  {
+    const int r = wave * 16 + l16;
+#pragma unroll
+    for (int kk = 0; kk < D / 32; ++kk)
+      qf[kk] = r < rows ? load_bf16x8(q + (size_t)(first + r / g) * q_stride + (size_t)(kvh * g + r % g) * D + kk * 32 + grp * 8)
+                        : zero_bf16x8();
+  }
+  // the rows whose scores and outputs this lane holds: 16 wave + 4 grp + r
+  int pr[4], lor[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + grp * 4 + r;
+    pr[r] = row < rows ? p_first + row / g : -1;
+    lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
+  }
+  float m_run[4], l_run[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY, l_run[r] = 0.f;
+  floatx4 o[DV / 16];
+#pragma unroll
+  for (int et = 0; et < DV / 16; ++et) o[et] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int kept_tiles = (kept + WAVE - 1) / WAVE;
+  const int first_window_tile = lo_first / WAVE > kept_tiles ? lo_first / WAVE : kept_tiles;
+  const int tiles = kept_tiles + (p_last / WAVE - first_window_tile + 1);
+  for (int ti = 0; ti < tiles; ++ti) {
+    const int j0 = (ti < kept_tiles ? ti : first_window_tile + (ti - kept_tiles)) * WAVE;
+    // scores of 16 rows x 64 keys: four 16-key tiles
+    floatx4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
+      const bool seen = j <= p_last && (j >= lo_first || j < kept);
+      const bf16* kp = seen ? kc + (((size_t)table[j / MFMA_PAGE] * Hkv + kvh) * MFMA_PAGE + (j % MFMA_PAGE)) * D + grp * 8 : nullptr;
+#pragma unroll
+      for (int kk = 0; kk < D / 32; ++kk) {
+        const bf16x8 kf = seen ? load_bf16x8(kp + kk * 32) : zero_bf16x8();
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], kf, s[t], 0, 0, 0);
+      }
+    }
+    // masks, running maxima and sums; the weights into the wave's LDS rows
+    float corr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float mx = -INFINITY;
+      bool ok[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int j = j0 + t * 16 + l16;
+        ok[t] = j <= pr[r] && (j >= lor[r] || j < keep_first);
+        s[t][r] = ok[t] ? s[t][r] * scale : -INFINITY;
+        mx = fmaxf(mx, s[t][r]);
+      }
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 16));
+      const float m_new = fmaxf(m_run[r], mx);
+      const bool none = m_new == -INFINITY;  // no key of this row so far
+      corr[r] = none ? 1.f : expf(m_run[r] - m_new);
+      float sum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float pj = (ok[t] && !none) ? expf(s[t][r] - m_new) : 0.f;
+        Pw[wave][grp * 4 + r][t * 16 + l16] = pj;
+        sum += pj;
+      }
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 16);
+      l_run[r] = l_run[r] * corr[r] + sum;
+      m_run[r] = m_new;
+    }
+#pragma unroll
+    for (int et = 0; et < DV / 16; ++et)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[et][r] *= corr[r];
+    __builtin_amdgcn_wave_barrier();  // a wave's own rows: its order of LDS operations is enough
+    // weights x values, 32 keys a step: row l16's weights of keys 32 ks + 8 grp .. + 7 in three bfloat16 pieces
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const float4 a0 = *reinterpret_cast<const float4*>(&Pw[wave][l16][ks * 32 + grp * 8]);
+      const float4 a1 = *reinterpret_cast<const float4*>(&Pw[wave][l16][ks * 32 + grp * 8 + 4]);
+      const float pv[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      bf16x8 hi, mid, low;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const bf16 h = static_cast<bf16>(pv[u]);
+        const float r1 = pv[u] - static_cast<float>(h);
+        const bf16 m = static_cast<bf16>(r1);
+        hi[u] = h;
+        mid[u] = m;
+        low[u] = static_cast<bf16>(r1 - static_cast<float>(m));
+      }
+      const int jb = j0 + ks * 32 + grp * 8;  // this lane's 8 keys as the B operand: one run of a page
+      int page = -1;
+      if (jb <= p_last && (jb + 8 > lo_first || jb < kept)) page = table[jb / MFMA_PAGE];
+      const bf16* vp = page >= 0 ? vc + ((size_t)page * Hkv + kvh) * DV * MFMA_PAGE + (jb % MFMA_PAGE) : nullptr;
+#pragma unroll
+      for (int et = 0; et < DV / 16; ++et) {
+        const bf16x8 vf = page >= 0 ? load_bf16x8(vp + (size_t)(et * 16 + l16) * MFMA_PAGE) : zero_bf16x8();
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf, o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, vf, o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, vf, o[et], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // the weights have been read before the next tile's are written
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + grp * 4 + r;
+    if (row >= rows) continue;
+    const float inv = 1.f / l_run[r];
+    bf16* ov = out + ((size_t)(first + row / g) * Hq + (kvh * g + row % g)) * DV;
+#pragma unroll
+    for (int et = 0; et < DV / 16; ++et) ov[et * 16 + l16] = static_cast<bf16>(o[et][r] * inv);
+  }
+}
+
+// 1 where the matrix-core form of the tiled kernel takes the shape (bfloat16 storage).
+extern "C" int ms_paged_attention_tiled_mfma_ok(int D, int Dv, int page_size) {
+  return page_size == MFMA_PAGE && (D == 32 || D == 64 || D == 96 || D == 128) && (Dv == 16 || Dv == 32 || Dv == 64 || Dv == 128);
+}
+
+// As ms_paged_attention_tiled for bfloat16 and the shapes above.
+extern "C" int ms_paged_attention_tiled_mfma(const void* q, int q_stride, const void* kc, const void* vc, const int* block_table,
+                                             int table_width, const int* tile_first, const int* tile_count, int tiles,
+                                             const int* token_row, const int* pos, void* out, int Hq, int Hkv, int D, int Dv,
+                                             int page_size, float scale, int window, int keep_first, hipStream_t st) {
+  if (tiles <= 0) return MS_OK;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || window < 0 || keep_first < 0 || table_width <= 0 || Hkv > 65535 || q_stride < Hq * D ||
+      q_stride % 8 || tile_first == nullptr || tile_count == nullptr)
+    return MS_BAD_ARG;
+  if (!ms_paged_attention_tiled_mfma_ok(D, Dv, page_size) || ms_paged_attention_tiled_tokens(Hq / Hkv, D, Dv) == 0) return MS_UNSUPPORTED;
+  if (window == 0) keep_first = 0;
+  dim3 grid(tiles, Hkv);
+#define TM(DD, EE)                                                                                                              \
+  paged_attention_tiled_mfma_kernel<DD, EE><<<grid, 256, 0, st>>>((const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, \
+                                                                  table_width, tile_first, tile_count, token_row, pos, (bf16*)out, Hq, \
+                                                                  Hkv, scale, window, keep_first)
+#define TD(DD)                      \
+  if (Dv == 16) TM(DD, 16);         \
+  else if (Dv == 32) TM(DD, 32);    \
+  else if (Dv == 64) TM(DD, 64);    \
+  else TM(DD, 128)
+  if (D == 32) { TD(32); }
+  else if (D == 64) { TD(64); }
+  else if (D == 96) { TD(96); }
+  else { TD(128); }
+#undef TD
+#undef TM
+  return launch_status();
+}

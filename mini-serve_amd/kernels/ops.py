@@ -59,6 +59,9 @@ _SIGNATURES = {
     "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
                                  _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
     "ms_paged_attention_tiled_tokens": [_c_int, _c_int, _c_int],
+    "ms_paged_attention_tiled_mfma": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
+                                      _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
+    "ms_paged_attention_tiled_mfma_ok": [_c_int, _c_int, _c_int],
     "ms_attention_decode_bf16": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void,
                                  _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_attention_decode_fused_bf16": [_c_void, _c_int, _c_ll, _c_void, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void,
@@ -680,8 +683,14 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
                    "paged_attention")
         if n_dec < t:
             first, count, tiles = _tiles_of(batch, tile_tokens, qkv.device)
-            _check(lib.ms_paged_attention_tiled(*generic, first.data_ptr(), count.data_ptr(), tiles, *meta, *shape, _stream()),
-                   "paged_attention_tiled")
+            if qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and lib.ms_paged_attention_tiled_mfma_ok(head_dim, dv, page):
+                # on the matrix cores, with every float32 softmax weight cut into three bfloat16 pieces: nothing is rounded
+                _check(lib.ms_paged_attention_tiled_mfma(qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common,
+                                                         first.data_ptr(), count.data_ptr(), tiles, *meta, *shape, _stream()),
+                       "paged_attention_tiled_mfma")
+            else:
+                _check(lib.ms_paged_attention_tiled(*generic, first.data_ptr(), count.data_ptr(), tiles, *meta, *shape, _stream()),
+                       "paged_attention_tiled")
         return out
     if n_dec:
         splits = decode_splits(n_dec, num_kv_heads, batch.max_kv_len)
