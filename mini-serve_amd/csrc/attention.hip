@@ -449,8 +449,9 @@ extern "C" int ms_paged_attention_tiled(const void* q, int q_stride, const void*
 // weight, not a rounding of it.
 //   A wave owns 16 of the block's 64 query rows. Scores: A = 16 query rows x 32 elements, B = 32 elements x 16 keys,
 //   both one 16-byte load per lane straight from global memory; a lane then holds one key of four rows
-//   (rows 4 (lane / 16) + r), a row's maximum and sum meet over the 16 lanes that share it. The weights go through a
-//   wave's own LDS rows to change hands (the second product wants a row's 8 consecutive keys in one lane); values:
+//   (rows 4 (lane / 16) + r), a row's maximum meets over the 16 lanes that share it; a row's sum of weights is one
+//   more column of the second product (values of 1), so it is the sum of exactly the pieces that meet the values.
+//   The weights go through a wave's own LDS rows to change hands (the second product wants a row's 8 consecutive keys in one lane); values:
 //   B = 32 keys x 16 elements, 8 consecutive tokens of one element being one 16-byte load from the transposed page.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -466,6 +467,16 @@ __device__ __forceinline__ bf16x8 zero_bf16x8() {
   x.u = make_uint4(0, 0, 0, 0);
   return x.v;
 }
+
+// Maximum over a row of 16 lanes, the same bits in all of them: four rotations within the row (DPP row_ror 8, 4, 2, 1).
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));
+  return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));
+}
+// e^x on the hardware's exp2 (about one unit in the last place, float32).
+__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 
 template <int D, int DV>
 __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
@@ -500,31 +511,51 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
     pr[r] = row < rows ? p_first + row / g : -1;
     lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
   }
-  float m_run[4], l_run[4];
+  float m_run[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY, l_run[r] = 0.f;
-  floatx4 o[DV / 16];
+  for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
+  floatx4 o[DV / 16], l_run = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int et = 0; et < DV / 16; ++et) o[et] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 ones;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) ones[u] = static_cast<bf16>(1.f);
 
   const int kept_tiles = (kept + WAVE - 1) / WAVE;
   const int first_window_tile = lo_first / WAVE > kept_tiles ? lo_first / WAVE : kept_tiles;
   const int tiles = kept_tiles + (p_last / WAVE - first_window_tile + 1);
   for (int ti = 0; ti < tiles; ++ti) {
     const int j0 = (ti < kept_tiles ? ti : first_window_tile + (ti - kept_tiles)) * WAVE;
+    // The tile's four pages (a tile of 64 keys is four whole pages; table rows are padded to a multiple of four
+    // entries): one load serves the keys' and the values' addresses.
+    const int4 pg4 = *reinterpret_cast<const int4*>(table + j0 / MFMA_PAGE);
+    const int pages[4] = {pg4.x, pg4.y, pg4.z, pg4.w};
+    // keys and values are asked for together, ahead of the first product: the values do not wait for the softmax
+    bf16x8 kf[4][D / 32], vf[2][DV / 16];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
+      const bool seen = j <= p_last && (j >= lo_first || j < kept) && pages[t] >= 0;
+      const bf16* kp = kc + (((size_t)(seen ? pages[t] : 0) * Hkv + kvh) * MFMA_PAGE + l16) * D + grp * 8;
+#pragma unroll
+      for (int kk = 0; kk < D / 32; ++kk) kf[t][kk] = seen ? load_bf16x8(kp + kk * 32) : zero_bf16x8();
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int jb = j0 + ks * 32 + grp * 8;  // this lane's 8 keys as the B operand: one run of a page
+      const int page = pages[ks * 2 + grp / 2];
+      const bool seen = jb <= p_last && (jb + 8 > lo_first || jb < kept) && page >= 0;
+      const bf16* vp = vc + ((size_t)(seen ? page : 0) * Hkv + kvh) * DV * MFMA_PAGE + (jb % MFMA_PAGE);
+#pragma unroll
+      for (int et = 0; et < DV / 16; ++et) vf[ks][et] = seen ? load_bf16x8(vp + (size_t)(et * 16 + l16) * MFMA_PAGE) : zero_bf16x8();
+    }
     // scores of 16 rows x 64 keys: four 16-key tiles
     floatx4 s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
-      const bool seen = j <= p_last && (j >= lo_first || j < kept);
-      const bf16* kp = seen ? kc + (((size_t)table[j / MFMA_PAGE] * Hkv + kvh) * MFMA_PAGE + (j % MFMA_PAGE)) * D + grp * 8 : nullptr;
 #pragma unroll
-      for (int kk = 0; kk < D / 32; ++kk) {
-        const bf16x8 kf = seen ? load_bf16x8(kp + kk * 32) : zero_bf16x8();
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], kf, s[t], 0, 0, 0);
-      }
+      for (int kk = 0; kk < D / 32; ++kk) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], kf[t][kk], s[t], 0, 0, 0);
     }
     // masks, running maxima and sums; the weights into the wave's LDS rows
     float corr[4];
@@ -539,21 +570,13 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
         s[t][r] = ok[t] ? s[t][r] * scale : -INFINITY;
         mx = fmaxf(mx, s[t][r]);
       }
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 16));
+      mx = row16_max(mx);
       const float m_new = fmaxf(m_run[r], mx);
       const bool none = m_new == -INFINITY;  // no key of this row so far
-      corr[r] = none ? 1.f : expf(m_run[r] - m_new);
-      float sum = 0.f;
+      corr[r] = none ? 1.f : exp_fast(m_run[r] - m_new);
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const float pj = (ok[t] && !none) ? expf(s[t][r] - m_new) : 0.f;
-        Pw[wave][grp * 4 + r][t * 16 + l16] = pj;
-        sum += pj;
-      }
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 16);
-      l_run[r] = l_run[r] * corr[r] + sum;
+      for (int t = 0; t < 4; ++t) Pw[wave][grp * 4 + r][t * 16 + l16] = (ok[t] && !none) ? exp_fast(s[t][r] - m_new) : 0.f;
+      l_run[r] *= corr[r];
       m_run[r] = m_new;
     }
 #pragma unroll
@@ -577,17 +600,15 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
         mid[u] = m;
         low[u] = static_cast<bf16>(r1 - static_cast<float>(m));
       }
-      const int jb = j0 + ks * 32 + grp * 8;  // this lane's 8 keys as the B operand: one run of a page
-      int page = -1;
-      if (jb <= p_last && (jb + 8 > lo_first || jb < kept)) page = table[jb / MFMA_PAGE];
-      const bf16* vp = page >= 0 ? vc + ((size_t)page * Hkv + kvh) * DV * MFMA_PAGE + (jb % MFMA_PAGE) : nullptr;
 #pragma unroll
       for (int et = 0; et < DV / 16; ++et) {
-        const bf16x8 vf = page >= 0 ? load_bf16x8(vp + (size_t)(et * 16 + l16) * MFMA_PAGE) : zero_bf16x8();
-        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf, o[et], 0, 0, 0);
-        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, vf, o[et], 0, 0, 0);
-        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, vf, o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf[ks][et], o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, vf[ks][et], o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, vf[ks][et], o[et], 0, 0, 0);
       }
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, ones, l_run, 0, 0, 0);
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, ones, l_run, 0, 0, 0);
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, ones, l_run, 0, 0, 0);
     }
     __builtin_amdgcn_wave_barrier();  // the weights have been read before the next tile's are written
   }

@@ -685,6 +685,10 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             first, count, tiles = _tiles_of(batch, tile_tokens, qkv.device)
             if qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and lib.ms_paged_attention_tiled_mfma_ok(head_dim, dv, page):
                 # on the matrix cores, with every float32 softmax weight cut into three bfloat16 pieces: nothing is rounded
+                if block_table.shape[1] % 4:  # the kernel reads the four page ids of a key tile at once
+                    wide = torch.zeros((block_table.shape[0], -(-block_table.shape[1] // 4) * 4), dtype=I32, device=block_table.device)
+                    wide[:, : block_table.shape[1]] = block_table
+                    common = (wide.data_ptr(), wide.shape[1])
                 _check(lib.ms_paged_attention_tiled_mfma(qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common,
                                                          first.data_ptr(), count.data_ptr(), tiles, *meta, *shape, _stream()),
                        "paged_attention_tiled_mfma")
