@@ -147,6 +147,7 @@ def plain_attention(q, k, v, scale, size, keep, groups):
     (2, 2, 8, 40, 6, "halves", 0, 0),        # every key visible
     (2, 1, 32, 32, 16, "adjacent", 45, 19),
     (2, 1, 128, 128, 32, "adjacent", 70, 9),   # the largest head the tiled kernel takes
+    (2, 1, 96, 16, 32, "adjacent", 30, 7),     # the matrix-core form's other sizes: keys of 96, values of 16
     (1, 1, 160, 136, 0, "halves", 50, 3),      # beyond it: the kernel with a wave (or several) per token and head
 ])
 def test_window_attention_with_kept_first_keys(H, G, D, E, rot, pairing, size, keep, dtype):
