@@ -13,9 +13,20 @@
 // (window == 0: all keys 0 .. p) and, with a window, the keys 0 .. keep_first - 1 as well (the
 // sequence's first tokens stay visible; tiles that hold neither kind of key are skipped, and their
 // pages are never read). Query head h reads KV head h / (Hq / Hkv).
+//
+// Options of the generic form (one wave, or several, per token and head):
+//   softcap > 0     a scaled score s becomes softcap * tanh(s / softcap);
+//   sinks           one float per query head whose exponential joins the softmax's denominator (it has no key and no
+//                   value, is neither scaled nor capped and counts once);
+//   value_share     this many consecutive key heads read the same value head (key head i: value head i / value_share;
+//                   the value cache then has Hkv / value_share heads): several score maps over one set of values;
+//   values_in_keys  the values are the first Dv elements of the key rows themselves (one vector per token serves as
+//                   key and as value); no value cache is read.
+// Head sizes up to 256, or, with at most eight waves, up to 1024.
 #include "common.h"
 
 #define MAX_HEAD_DIM 256
+#define MAX_WIDE_HEAD_DIM 1024
 
 template <typename T> struct Vec16;  // 16 bytes of T
 template <> struct Vec16<float> { static constexpr int N = 4; };
@@ -24,21 +35,23 @@ template <> struct Vec16<bf16> { static constexpr int N = 8; };
 // NW waves per (token, query head): wave w visits the tiles number w, w + NW, ... of those that hold visible keys,
 // and the waves' running maxima, sums and outputs meet in LDS in wave order. NW == 1 is the plain form; more waves
 // serve steps of few tokens (decode), where one wave per head would walk a long window alone.
-template <typename T, int NW>
+template <typename T, int NW, int MAXD>
 __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ kc, const T* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ token_list,
     const int* __restrict__ token_row, const int* __restrict__ pos, T* __restrict__ out, int Hq, int Hkv, int D, int Dv,
-    int page_size, float scale, int window, int keep_first) {
-  __shared__ __attribute__((aligned(16))) float qs[MAX_HEAD_DIM];
+    int page_size, float scale, int window, int keep_first, float softcap, const float* __restrict__ sinks, int value_share,
+    int values_in_keys) {
+  __shared__ __attribute__((aligned(16))) float qs[MAXD];
   __shared__ float ps[NW][WAVE];
   __shared__ float ml[NW][2];
-  __shared__ float os[NW > 1 ? NW : 1][NW > 1 ? MAX_HEAD_DIM : 1];
+  __shared__ float os[NW > 1 ? NW : 1][NW > 1 ? MAXD : 1];
   constexpr int VN = Vec16<T>::N;
-  constexpr int PER = MAX_HEAD_DIM / WAVE;
+  constexpr int PER = MAXD / WAVE;
   const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int kvh = h / (Hq / Hkv);
+  const int Hv = Hkv / value_share, vh = kvh / value_share;  // the value head this key head's scores weigh
   const int p = pos[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int kept = keep_first < lo ? keep_first : lo;  // keys 0 .. kept - 1 are visible beside lo .. p
@@ -78,6 +91,7 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
         for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(kp[d]), dot);
       }
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m_run, wave_max(s));  // finite: every visited tile holds a visible key
     const float pj = valid ? expf(s - m_new) : 0.f;
@@ -91,7 +105,30 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] *= corr;
     const int je = j0 + WAVE - 1 < p ? j0 + WAVE - 1 : p;
-    if (page_size % VN == 0 && WAVE % page_size == 0) {
+    if (values_in_keys) {
+      // Key by key: the lanes read a run of the key's own row, four keys' loads under way at a time.
+      for (int jj = j0; jj <= je; jj += 4) {
+        float w[4];
+        const T* vp[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int ju = jj + u;
+          const bool seen = ju <= je && (ju >= lo || ju < kept);
+          w[u] = seen ? ps[wave][ju - j0] : 0.f;
+          vp[u] = seen ? kc + (((size_t)table[ju / page_size] * Hkv + kvh) * page_size + (ju % page_size)) * D : nullptr;
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int e = lane + i * WAVE;
+          if (e >= Dv) continue;
+          float vv[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) vv[u] = vp[u] ? to_f32(vp[u][e]) : 0.f;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) o[i] = fmaf(w[u], vv[u], o[i]);
+        }
+      }
+    } else if (page_size % VN == 0 && WAVE % page_size == 0) {
       // Page by page: a lane fetches the page's tokens of its element as 16-byte runs (the page keeps the tokens of
       // one element side by side). Keys that are not visible carry the weight 0, and fmaf(0, v, o) is o: the sum is
       // the one over the visible keys in ascending order. Pages that were given back are not read.
@@ -99,7 +136,7 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
         if (jp + page_size <= lo && jp >= kept) continue;  // wholly in the gap
         const int page = table[jp / page_size];
         if (page < 0) continue;
-        const T* vp = vc + ((size_t)page * Hkv + kvh) * Dv * page_size;
+        const T* vp = vc + ((size_t)page * Hv + vh) * Dv * page_size;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
           const int e = lane + i * WAVE;
@@ -119,7 +156,7 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
           continue;
         }
         const int page = table[jj / page_size];
-        const T* vp = vc + ((size_t)page * Hkv + kvh) * Dv * page_size + (jj % page_size);
+        const T* vp = vc + ((size_t)page * Hv + vh) * Dv * page_size + (jj % page_size);
         const float w = ps[wave][jj - j0];
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -144,6 +181,7 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
     float m_all = ml[0][0];  // wave 0 always has a tile
 #pragma unroll
     for (int w = 1; w < NW; ++w) m_all = fmaxf(m_all, ml[w][0]);
+    m_run = m_all;
     l_run = 0.f;
 #pragma unroll
     for (int i = 0; i < PER; ++i) o[i] = 0.f;
@@ -159,7 +197,13 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
     }
   }
   T* ov = out + ((size_t)t * Hq + h) * Dv;
-  const float inv = 1.f / l_run;
+  float inv = 1.f / l_run;
+  if (sinks) {
+    // exp(sink) joins the denominator: both are brought to the larger of the two maxima first
+    const float sink = sinks[h], m_all = fmaxf(m_run, sink);
+    const float c = expf(m_run - m_all);
+    inv = c / (l_run * c + expf(sink - m_all));
+  }
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + i * WAVE;
@@ -171,21 +215,32 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
                                           const int* block_table, int table_width, const int* token_list,
                                           const int* token_row, const int* pos, void* out, int tokens, int Hq, int Hkv,
                                           int D, int Dv, int page_size, float scale, int window, int keep_first, int waves,
+                                          float softcap, const float* sinks, int value_share, int values_in_keys,
                                           hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (D <= 0 || D > MAX_HEAD_DIM || Dv <= 0 || Dv > MAX_HEAD_DIM || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 ||
-      window < 0 || keep_first < 0 || table_width <= 0 || Hq > 65535 || q_stride < Hq * D || (waves != 1 && waves != 8 && waves != 16))
+  if (D <= 0 || D > MAX_WIDE_HEAD_DIM || Dv <= 0 || Dv > MAX_WIDE_HEAD_DIM || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 ||
+      window < 0 || keep_first < 0 || table_width <= 0 || Hq > 65535 || q_stride < Hq * D || (waves != 1 && waves != 8 && waves != 16) ||
+      !(softcap >= 0.f) || value_share < 1 || Hkv % value_share || (values_in_keys && (Dv > D || value_share != 1)) ||
+      (!values_in_keys && vc == nullptr))
     return MS_BAD_ARG;
   if (window == 0) keep_first = 0;  // every key is visible anyway
+  const bool wide = D > MAX_HEAD_DIM || Dv > MAX_HEAD_DIM;
+  if (wide && waves == 16) waves = 8;  // the waves' partial outputs must fit in LDS
   dim3 grid(tokens, Hq);
-#define GA(T, NW)                                                                                                           \
-  paged_attention_generic_kernel<T, NW><<<grid, NW * WAVE, 0, st>>>((const T*)q, q_stride, (const T*)kc, (const T*)vc, block_table, \
-                                                                    table_width, token_list, token_row, pos, (T*)out, Hq, Hkv, D, Dv, \
-                                                                    page_size, scale, window, keep_first)
-  if (is_bf16) {
-    if (waves == 16) GA(bf16, 16); else if (waves == 8) GA(bf16, 8); else GA(bf16, 1);
+#define GA(T, NW, MAXD)                                                                                                      \
+  paged_attention_generic_kernel<T, NW, MAXD><<<grid, NW * WAVE, 0, st>>>(                                                   \
+      (const T*)q, q_stride, (const T*)kc, (const T*)vc, block_table, table_width, token_list, token_row, pos, (T*)out, Hq, Hkv, D, \
+      Dv, page_size, scale, window, keep_first, softcap, sinks, value_share, values_in_keys)
+  if (wide) {
+    if (is_bf16) {
+      if (waves == 8) GA(bf16, 8, MAX_WIDE_HEAD_DIM); else GA(bf16, 1, MAX_WIDE_HEAD_DIM);
+    } else {
+      if (waves == 8) GA(float, 8, MAX_WIDE_HEAD_DIM); else GA(float, 1, MAX_WIDE_HEAD_DIM);
+    }
+  } else if (is_bf16) {
+    if (waves == 16) GA(bf16, 16, MAX_HEAD_DIM); else if (waves == 8) GA(bf16, 8, MAX_HEAD_DIM); else GA(bf16, 1, MAX_HEAD_DIM);
   } else {
-    if (waves == 16) GA(float, 16); else if (waves == 8) GA(float, 8); else GA(float, 1);
+    if (waves == 16) GA(float, 16, MAX_HEAD_DIM); else if (waves == 8) GA(float, 8, MAX_HEAD_DIM); else GA(float, 1, MAX_HEAD_DIM);
   }
 #undef GA
   return launch_status();

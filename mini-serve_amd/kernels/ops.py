@@ -55,7 +55,16 @@ _SIGNATURES = {
     "ms_gemm_bf16_small_tile_cols": [_c_int, _c_int],
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
-                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_void],
+                                   _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int,
+                                   _c_float, _c_void, _c_int, _c_int, _c_void],
+    "ms_conv_norm_store": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                           _c_void, _c_float, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                           _c_int, _c_int, _c_int, _c_void],
+    "ms_map_difference_norm": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void],
+    "ms_latent_prepare": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_int, _c_float, _c_void, _c_void,
+                          _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_activate": [_c_void, _c_void, _c_int, _c_ll, _c_int, _c_void],
     "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
                                  _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void],
     "ms_paged_attention_tiled_tokens": [_c_int, _c_int, _c_int],
@@ -535,6 +544,29 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, value_dim: in
     return page
 
 
+GENERIC_MAX_HEAD_DIM = 1024  # head sizes the generic attention kernel takes (MAX_WIDE_HEAD_DIM in csrc/attention.hip)
+
+
+def _check_special_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, value_dim, value_share, values_in_keys) -> int:
+    """Keys ``[pages, Hkv, page, D]``; values ``[pages, Hkv / value_share, Dv, page]``, or none where the keys' rows
+    hold them. Returns the page size."""
+    _dev(k_cache, "k_cache", dtype, 4)
+    page = k_cache.shape[2]
+    if tuple(k_cache.shape[1:]) != (num_kv_heads, page, head_dim):
+        raise ValueError(f"k_cache is {tuple(k_cache.shape)}, expected [pages, {num_kv_heads}, page, {head_dim}]")
+    if value_share < 1 or num_kv_heads % value_share:
+        raise ValueError(f"{num_kv_heads} key heads cannot share values in runs of {value_share}")
+    if values_in_keys:
+        if v_cache is not None or value_share != 1 or value_dim > head_dim:
+            raise ValueError("values inside the keys: no value cache, no sharing, and a value size up to the key size")
+        return page
+    _dev(v_cache, "v_cache", dtype, 4)
+    want = (k_cache.shape[0], num_kv_heads // value_share, value_dim, page)
+    if tuple(v_cache.shape) != want:
+        raise ValueError(f"v_cache is {tuple(v_cache.shape)}, expected {list(want)}")
+    return page
+
+
 PREFILL_BIG_BLOCKS = 640  # from this many 128-row blocks on, the prefill attention runs 128-row blocks
 DECODE_TARGET_BLOCKS = 512  # workgroups the split decode kernel aims for
 DECODE_MIN_CHUNKS = 4  # 32-token chunks a split should at least hold
@@ -632,7 +664,8 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
 
 
 def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window,
-                    value_dim: int | None = None, keep_first: int = 0, exact_weights: bool = False):
+                    value_dim: int | None = None, keep_first: int = 0, exact_weights: bool = False, softcap: float = 0.0,
+                    sinks: torch.Tensor | None = None, value_share: int = 1, values_in_keys: bool = False):
     """Attention of the batch's new tokens over the cache. ``qkv [T, >= Hq D]`` holds the queries
     in its first ``Hq * D`` columns. Returns ``[T, Hq * Dv]`` (``Dv = D`` unless ``value_dim`` is given).
     A query at position p sees keys ``max(0, p - window + 1) .. p`` (``window == 0``: all up to p) and, with a
@@ -641,13 +674,30 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     bfloat16 with 16-token pages and a head size of 64 or 128: rows that bring one token run the
     split decode kernel, rows that bring several the tiled prefill kernel. Everything else (float32,
     other head sizes or page sizes, values of another size than the keys, kept first keys, or
-    ``exact_weights``: softmax weights that must meet the values unrounded) runs the generic kernel."""
+    ``exact_weights``: softmax weights that must meet the values unrounded) runs the generic kernel.
+
+    Options that only the generic kernel knows (float32 arithmetic throughout, head sizes up to 1024):
+    ``softcap > 0`` bounds a scaled score ``s`` to ``softcap * tanh(s / softcap)``; ``sinks`` (float32 ``[Hq]``) adds
+    ``exp(sinks[h])`` to head ``h``'s softmax denominator; ``value_share = n`` lets ``n`` consecutive key heads weigh
+    the same value head (``v_cache`` then has ``Hkv / n`` heads); ``values_in_keys`` takes the first ``Dv`` elements
+    of each key row as that token's value (``v_cache`` is None)."""
     _dev(qkv, "qkv", (F32, BF16), 2)
     t = qkv.shape[0]
     dv = head_dim if value_dim is None else int(value_dim)
-    page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, dv)
-    if not (1 <= head_dim <= 256 and 1 <= dv <= 256):
-        raise ValueError(f"head sizes {head_dim} / {dv} are not supported: the attention kernels take sizes up to 256")
+    special = bool(softcap) or sinks is not None or value_share != 1 or values_in_keys
+    if special:
+        page = _check_special_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, dv, value_share, values_in_keys)
+        if sinks is not None:
+            _dev(sinks, "sinks", F32, 1)
+            if sinks.shape[0] != num_heads:
+                raise ValueError(f"{sinks.shape[0]} sinks for {num_heads} query heads")
+        if not softcap >= 0:
+            raise ValueError(f"softcap must not be negative, got {softcap}")
+    else:
+        page = _check_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, dv)
+    limit = GENERIC_MAX_HEAD_DIM if special else 256
+    if not (1 <= head_dim <= limit and 1 <= dv <= limit):
+        raise ValueError(f"head sizes {head_dim} / {dv} are not supported: the attention kernels take sizes up to {limit}")
     if keep_first < 0 or window < 0:
         raise ValueError("window and keep_first must not be negative")
     if num_heads % num_kv_heads:
@@ -667,20 +717,32 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     meta = (batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr())
     n_dec = batch.num_decode_tokens
     fast = (qkv.dtype == BF16 and page == 16 and head_dim in (64, 128) and num_heads // num_kv_heads <= 16
-            and qkv.shape[1] % 8 == 0 and dv == head_dim and not (window and keep_first) and not exact_weights)
+            and qkv.shape[1] % 8 == 0 and dv == head_dim and not (window and keep_first) and not exact_weights and not special)
     if not fast:
-        generic = (qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), int(qkv.dtype == BF16), *common)
+        generic = (qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), _ptr(v_cache), int(qkv.dtype == BF16), *common)
         shape = (num_heads, num_kv_heads, head_dim, dv, page, float(scale), int(window), int(keep_first))
-        tile_tokens = lib.ms_paged_attention_tiled_tokens(num_heads // num_kv_heads, head_dim, dv)
+        extra = (float(softcap), _ptr(sinks), int(value_share), int(values_in_keys))
+        tile_tokens = 0 if special else lib.ms_paged_attention_tiled_tokens(num_heads // num_kv_heads, head_dim, dv)
         lens = getattr(batch, "row_lens", None)
+        if special and lens is not None and 0 < n_dec < t:
+            # single-token rows walk their keys with several waves, the others with one wave per token and head
+            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES,
+                                                  *extra, _stream()), "paged_attention")
+            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.prefill_tokens), *meta, t - n_dec, *shape, 1, *extra,
+                                                  _stream()), "paged_attention")
+            return out
+        if special and lens is not None and n_dec == t:
+            _check(lib.ms_paged_attention_generic(*generic, None, *meta, t, *shape, DECODE_GENERIC_WAVES, *extra, _stream()),
+                   "paged_attention")
+            return out
         if not (exact_weights or keep_first or dv != head_dim) or not tile_tokens or lens is None:
             # the form whose sums have one order whatever the step looks like: float32 results stay bitwise equal
-            _check(lib.ms_paged_attention_generic(*generic, None, *meta, t, *shape, 1, _stream()), "paged_attention")
+            _check(lib.ms_paged_attention_generic(*generic, None, *meta, t, *shape, 1, *extra, _stream()), "paged_attention")
             return out
         # rows that bring one token: several waves share a head's keys; rows that bring several: tiles of tokens in LDS
         if n_dec:
-            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES, _stream()),
-                   "paged_attention")
+            _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES,
+                                                  *extra, _stream()), "paged_attention")
         if n_dec < t:
             first, count, tiles = _tiles_of(batch, tile_tokens, qkv.device)
             if qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and lib.ms_paged_attention_tiled_mfma_ok(head_dim, dv, page):
@@ -966,6 +1028,166 @@ def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_ca
         _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, int(value_dim), page_size, _stream()),
         "qkv_norm_rope_store")
     return q_out
+
+
+# ------------------------------------------------------------------------------------- between projection and attention
+
+
+def conv_norm_store(x, conv_weight, taps: int, state, batch, q_weight, k_weight, eps, slots, k_cache, v_cache, q_groups: int,
+                    k_groups: int, value_heads: int, head_dim: int, value_dim: int, out_dtype) -> torch.Tensor:
+    """A short causal convolution over time on every channel of the float32 projection ``x [T, q_groups D + k_groups D +
+    value_heads Dv]`` (``conv_weight [channels, taps]``; ``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zero before a
+    sequence's start), an RMS norm over every group of ``D`` query and key channels (weights ``[D]``, shared by the
+    groups; None: no norm), then the store: keys ``[pages, k_groups, page, D]`` and values ``[pages, value_heads, Dv,
+    page]`` at ``slots``. Returns the queries ``[T, q_groups D]`` in ``out_dtype``.
+
+    ``state`` (float32 ``[slots + 1, taps - 1, channels]``) holds each request's last ``taps - 1`` projection rows:
+    row ``batch.state_slots[b]`` feeds the positions before this step and is brought up to date afterwards. A request
+    that starts at position 0 reads nothing of it."""
+    _dev(x, "x", F32, 2)
+    t = x.shape[0]
+    channels = (q_groups + k_groups) * head_dim + value_heads * value_dim
+    if x.shape[1] != channels:
+        raise ValueError(f"x has width {x.shape[1]}, expected {channels}")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    _dev(conv_weight, "conv_weight", (F32, BF16), 2)
+    if tuple(conv_weight.shape) != (channels, taps) or taps < 1:
+        raise ValueError(f"conv_weight is {tuple(conv_weight.shape)}, expected [{channels}, {taps}]")
+    if (q_weight is None) != (k_weight is None):
+        raise ValueError("the query and the key norm come together or not at all")
+    for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
+        if w is not None:
+            _dev(w, nm, conv_weight.dtype, 1)
+            if w.shape[0] != head_dim:
+                raise ValueError(f"{nm} weight has {w.shape[0]} elements, expected {head_dim}")
+    if taps > 1:
+        _dev(state, "state", F32, 3)
+        if tuple(state.shape[1:]) != (taps - 1, channels):
+            raise ValueError(f"state is {tuple(state.shape)}, expected [slots, {taps - 1}, {channels}]")
+    _dev(slots, "slots", I32, 1)
+    for name in ("token_row", "positions"):
+        _dev(getattr(batch, name), name, I32, 1)
+        if getattr(batch, name).shape[0] != t:
+            raise ValueError("batch metadata does not match the number of tokens")
+    if slots.shape[0] != t or batch.row_start.shape[0] < batch.num_rows + 1:
+        raise ValueError("one slot per token and one start per row are needed")
+    page = _check_special_caches(k_cache, v_cache, out_dtype, k_groups, head_dim, value_dim, k_groups // value_heads, False)
+    q_out = torch.empty((t, q_groups * head_dim), dtype=out_dtype, device=x.device)
+    _check(library().ms_conv_norm_store(
+        x.data_ptr(), x.shape[1], conv_weight.data_ptr(), int(conv_weight.dtype == BF16), int(taps), _ptr(state) if taps > 1 else None,
+        batch.state_slots.data_ptr(), batch.token_row.data_ptr(), batch.positions.data_ptr(), batch.row_start.data_ptr(),
+        batch.starts.data_ptr(), _ptr(q_weight), _ptr(k_weight), float(eps), q_out.data_ptr(), slots.data_ptr(), k_cache.data_ptr(),
+        v_cache.data_ptr(), int(out_dtype == BF16), t, batch.num_rows, q_groups, k_groups, value_heads, head_dim, value_dim, page,
+        _stream()), "conv_norm_store")
+    return q_out
+
+
+def map_difference_norm(a: torch.Tensor, groups: int, per_group: int, value_dim: int, weight: float, eps: float,
+                        out_scale: float) -> torch.Tensor:
+    """``a [T, groups * 2 * per_group * Dv]`` holds two attention maps' outputs per head, ordered (group, map, head of
+    the group). Per head: ``o = a1 - weight * a2``, divided by its root mean square over ``Dv`` (``eps`` inside the
+    root), times ``out_scale``. Returns ``[T, groups * per_group * Dv]`` in ``a``'s dtype, float32 arithmetic."""
+    _dev(a, "a", (F32, BF16), 2)
+    if a.shape[1] != groups * 2 * per_group * value_dim:
+        raise ValueError(f"a has width {a.shape[1]}, expected {groups * 2 * per_group * value_dim}")
+    out = torch.empty((a.shape[0], groups * per_group * value_dim), dtype=a.dtype, device=a.device)
+    _check(library().ms_map_difference_norm(a.data_ptr(), out.data_ptr(), int(a.dtype == BF16), a.shape[0], groups, per_group,
+                                            value_dim, float(weight), float(eps), float(out_scale), _stream()), "map_difference_norm")
+    return out
+
+
+def latent_prepare(x, q_col: int, kv_col: int | None, rope, rot: int, pairing: str, latent_weight, eps, slots, k_cache,
+                   heads: int, plain_dim: int, rot_dim: int, latent_dim: int, out_dtype):
+    """From the float32 projection ``x``: every head's plain query part into ``q_plain [T, H Dn]``, its turned part into
+    the last ``R`` columns of that head in ``q_full [T, H (C + R)]`` (the first ``C`` are left for the caller), and, with
+    ``kv_col``, the token's cache row ``[C + R]`` at ``slots``: the latent after an RMS norm (``latent_weight``) and the
+    turned shared key part. The first ``rot`` of the ``R`` elements turn by ``rope``'s angles. Returns ``(q_plain, q_full)``."""
+    _dev(x, "x", F32, 2)
+    t = x.shape[0]
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    if rot:
+        _dev(rope, "rope", F32, 2)
+        if tuple(rope.shape) != (t, rot):
+            raise ValueError(f"rotation table is {tuple(rope.shape)}, expected [{t}, {rot}]")
+    w_bf16 = 0
+    if kv_col is not None:
+        _dev(slots, "slots", I32, 1)
+        _dev(k_cache, "k_cache", out_dtype, 4)
+        _dev(latent_weight, "latent_weight", (F32, BF16), 1)
+        if slots.shape[0] != t or tuple(k_cache.shape[1:]) != (1, k_cache.shape[2], latent_dim + rot_dim) or latent_weight.shape[0] != latent_dim:
+            raise ValueError("one slot per token, a cache of one head of C + R elements and a weight of C elements are needed")
+        w_bf16 = int(latent_weight.dtype == BF16)
+    q_plain = torch.empty((t, heads * plain_dim), dtype=out_dtype, device=x.device)
+    q_full = torch.empty((t, heads * (latent_dim + rot_dim)), dtype=out_dtype, device=x.device)
+    _check(library().ms_latent_prepare(
+        x.data_ptr(), x.shape[1], int(q_col), -1 if kv_col is None else int(kv_col), _ptr(rope) if rot else None, int(rot),
+        _pairing(pairing), _ptr(latent_weight) if kv_col is not None else None, w_bf16, float(eps), q_plain.data_ptr(),
+        q_full.data_ptr(), _ptr(slots) if kv_col is not None else None, _ptr(k_cache) if kv_col is not None else None,
+        int(out_dtype == BF16), t, heads, plain_dim, rot_dim, latent_dim, _stream()), "latent_prepare")
+    return q_plain, q_full
+
+
+def head_gate_(o: torch.Tensor, x: torch.Tensor, col: int, heads: int) -> torch.Tensor:
+    """``o[t, h, :] *= sigmoid(x[t, col + h])`` in place: ``o [T, heads * E]``, ``x`` float32."""
+    _dev(o, "o", (F32, BF16), 2)
+    _dev(x, "x", F32, 2)
+    if o.shape[0] != x.shape[0] or o.shape[1] % heads or x.shape[1] < col + heads:
+        raise ValueError("o and x must have the same rows, and x one gate column per head")
+    _check(library().ms_head_gate(o.data_ptr(), int(o.dtype == BF16), x.data_ptr(), x.shape[1], int(col), o.shape[0], heads,
+                                  o.shape[1] // heads, _stream()), "head_gate")
+    return o
+
+
+def activate(x: torch.Tensor, activation: str, out_dtype) -> torch.Tensor:
+    """``act(x)`` elementwise for a feed-forward without a gate: float32 in, ``out_dtype`` out, float32 arithmetic."""
+    _dev(x, "x", F32)
+    if activation not in ACTIVATIONS or activation in ACTIVATIONS_WITH_LIMIT:
+        raise NotImplementedError(f"activation {activation!r} has no ungated form here")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _check(library().ms_activate(x.data_ptr(), out.data_ptr(), int(out_dtype == BF16), x.numel(), ACTIVATIONS[activation], _stream()),
+           "activate")
+    return out
+
+
+def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_col: int = 0) -> torch.Tensor:
+    """A matrix product per head: ``out[:, h * stride + out_col : ... + N] = x[:, h * K : (h + 1) * K] @ weights[h]^T`` with
+    ``x [M, H K]``, ``weights [H, N, K]`` and ``out [M, H stride]`` (``stride = out.shape[1] / H >= out_col + N``; the other
+    columns of ``out`` stay). One launch of the engine's matrix kernels per head, over strided rows. Where a head's slice
+    does not start at a multiple of 16 bytes the head goes through contiguous copies."""
+    _dev(x, "x", (F32, BF16), 2)
+    _dev(weights, "weights", (F32, BF16), 3)
+    _dev(out, "out", (F32, BF16), 2)
+    h, n, k = weights.shape
+    m = x.shape[0]
+    if x.shape[1] != h * k or out.shape[0] != m or out.shape[1] % h or out.shape[1] // h < out_col + n:
+        raise ValueError(f"head_linear: x {tuple(x.shape)}, weights {tuple(weights.shape)}, out {tuple(out.shape)} at column {out_col}")
+    if m == 0:
+        return out
+    stride = out.shape[1] // h
+    lib = library()
+    f32 = weights.dtype == F32
+    xa = cast(x, F32 if f32 else BF16)
+    xi, oi = xa.element_size(), out.element_size()
+    # the matrix-core kernels fetch 16 bytes at a time and store up to 16: every head's slices must start at such a multiple
+    direct = f32 or (k % 8 == 0 and (stride * oi) % 16 == 0 and (out_col * oi) % 16 == 0)
+    if not direct:
+        for i in range(h):
+            y = linear(xa[:, i * k : (i + 1) * k].contiguous(), weights[i], out_dtype=out.dtype)
+            out[:, i * stride + out_col : i * stride + out_col + n].copy_(y)
+        return out
+    for i in range(h):
+        xp = xa.data_ptr() + i * k * xi
+        wp = weights.data_ptr() + i * n * k * weights.element_size()
+        op = out.data_ptr() + (i * stride + out_col) * oi
+        if f32:
+            _check(lib.ms_gemm_f32(xp, wp, op, 0 if out.dtype == F32 else 2, m, n, k, h * k, out.shape[1], _stream()), "gemm_f32")
+        else:
+            _check(lib.ms_gemm_bf16(xp, wp, op, 1 if out.dtype == F32 else 0, m, n, k, h * k, out.shape[1], 1, _stream()), "gemm_bf16")
+    return out
 
 
 # ------------------------------------------------------------------------------------- linear recurrences

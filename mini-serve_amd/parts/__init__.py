@@ -1,4 +1,4 @@
-from . import attention, block, embedding, mlp, norm, recurrent, rotary  # noqa: F401  (register the built-in parts)
+from . import attention, attention_forms, block, embedding, mlp, norm, recurrent, rotary  # noqa: F401  (register the built-in parts)
 from .base import (
     Block, CachePlane, Embedding, FeedForward, Head, KVNeed, Mixer, Norm, Part, PositionEncoding, Rotation,
     Runtime, StateNeed, StateTensor, TensorSpec,

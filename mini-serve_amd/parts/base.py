@@ -39,12 +39,14 @@ class TensorSpec:
     ``init`` says how the random-weights mode draws it: ``"normal"`` N(0, std) (matrices, embeddings),
     ``"ones"`` a scale around one (norm weights: all one, or uniform in the range the caller gives),
     ``"uniform"`` U(-std, std), ``"zeros"`` (a bias that starts switched off); integer tables are
-    drawn uniformly from ``[0, high)``."""
+    drawn uniformly from ``[0, high)``. ``optional``: a checkpoint may hold the tensor or not; nothing reads it
+    (the loader accepts it, the random-weights mode does not draw it, the part is not handed it)."""
 
     shape: tuple[int, ...]
     kind: str = "float"
     init: str = "normal"
     high: int | None = None
+    optional: bool = False
 
     def __post_init__(self):
         if self.kind not in ("float", "int"):
@@ -185,6 +187,11 @@ class Norm(Part):
         """Normalise rows of the float32 ``x`` plus ``add`` (a pending sum). Without ``rows``, ``x`` is
         also brought up to date in place; with ``rows`` the stream is not read again and stays as it is."""
         raise NotImplementedError
+
+    def add_normed(self, residual, stream) -> None:
+        """``residual += norm(stream)`` row by row, both float32 and of one shape: the norm of a layer that norms
+        what a sublayer puts out instead of what it reads."""
+        raise NotImplementedError(f"norm {self.kind!r} cannot norm a sublayer's output into the residual stream")
 
 
 class PositionEncoding(Part):

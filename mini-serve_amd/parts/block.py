@@ -1,8 +1,10 @@
 """Block arrangements: where the norms and the residual sums sit around a mixer and a
 feed-forward. ``prenorm`` is the reference's (miniserve/model/qwen3.py:212-216):
-``h += mixer(norm(h)); h += feed_forward(norm(h))``."""
+``h += mixer(norm(h)); h += feed_forward(norm(h))``. ``parallel`` and ``outnorm`` have no counterpart there."""
 
 from __future__ import annotations
+
+import torch
 
 from ..config.spec import PartSpec
 from .base import Block, TensorSpec
@@ -66,3 +68,49 @@ class ParallelBlock(Block):
 
     def parameters_bytes(self) -> int:
         return self.norm.parameters_bytes()
+
+
+@register("block", "outnorm")
+class OutputNormBlock(Block):
+    """``h += norm1(mixer(h)); h += norm2(feed_forward(h))``: the sublayers read the stream itself, and what they put
+    out is normed before it joins the stream. Each sublayer adds into a stream of its own that starts at zero; the
+    norm's ``add_normed`` folds it into the residual stream. A layer without a feed-forward has no second norm
+    (``ffn_norm`` None); ``spare`` then names norm tensors ``{name: width}`` that a checkpoint may still carry for it."""
+
+    def __init__(self, spec: PartSpec, rt, mixer, feed_forward):
+        super().__init__(spec, rt, mixer, feed_forward)
+        mn, fn = spec["mixer_norm"], spec.get("ffn_norm")
+        self.mixer_norm = part_class("norm", mn)(mn, rt)
+        self.ffn_norm = part_class("norm", fn)(fn, rt) if fn is not None else None
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        out = {}
+        for key in ("mixer_norm", "ffn_norm"):
+            s = spec.get(key)
+            if s is not None:
+                out.update(part_class("norm", s).tensors(s))
+        for name, width in (spec.get("spare") or {}).items():
+            out[name] = TensorSpec((int(width),), optional=True)
+        return out
+
+    def bind(self, tensors) -> None:
+        self.mixer_norm.bind(tensors)
+        if self.ffn_norm is not None:
+            self.ffn_norm.bind(tensors)
+
+    def _sublayer(self, run, norm, residual) -> None:
+        ops = self.rt.ops
+        own = torch.zeros_like(residual)
+        ops.add_pending(own, run(ops.cast(residual, self.rt.dtype), own))
+        norm.add_normed(residual, own)
+
+    def forward(self, residual, batch, cache, state, pending=None):
+        self.rt.ops.add_pending(residual, pending)
+        self._sublayer(lambda x, own: self.mixer.forward(x, batch, cache, state, own), self.mixer_norm, residual)
+        if self.ffn_norm is not None:
+            self._sublayer(lambda x, own: self.feed_forward.forward(x, own), self.ffn_norm, residual)
+        return None
+
+    def parameters_bytes(self) -> int:
+        return self.mixer_norm.parameters_bytes() + (self.ffn_norm.parameters_bytes() if self.ffn_norm is not None else 0)

@@ -7,7 +7,9 @@ once; the down projection adds into the residual stream in its epilogue.
 
 ``names`` (optional) maps ``gate`` / ``up`` / ``down`` to the tensors' names behind the prefix (default
 ``<x>_proj.weight``); ``limit`` belongs to the activations that bound their inputs (``swiglu_clamped``).
-``none`` is the feed-forward of a layer that has none."""
+``none`` is the feed-forward of a layer that has none. ``dense_mlp`` (no counterpart in the reference) is
+``down(act(up(x)))`` without a gate: tensors ``up`` / ``down`` (``names``), the activation in float32 on the float32
+result of the first product, rounded once."""
 
 from __future__ import annotations
 
@@ -73,3 +75,38 @@ class GatedMLP(FeedForward):
 
     def flops(self, rows) -> int:
         return 2 * sum(n for n, _ in rows) * 3 * self.hidden * self.inter
+
+
+@register("feed_forward", "dense_mlp")
+class DenseMLP(FeedForward):
+    def __init__(self, spec: PartSpec, rt):
+        super().__init__(spec, rt)
+        self.prefix = spec.get("prefix", "")
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.activation = spec.get("activation", "gelu_tanh")
+        if rt is not None and (self.activation not in rt.ops.ACTIVATIONS or self.activation in rt.ops.ACTIVATIONS_WITH_LIMIT):
+            raise NotImplementedError(f"activation {self.activation!r} has no ungated form")
+        given = spec.get("names") or {}
+        self.names = {k: self.prefix + given.get(k, f"{k}_proj.weight") for k in ("up", "down")}
+        self.up = self.down = None
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        h, i, p = int(spec["hidden_size"]), int(spec["intermediate_size"]), spec.get("prefix", "")
+        given = spec.get("names") or {}
+        return {p + given.get("up", "up_proj.weight"): TensorSpec((i, h)), p + given.get("down", "down_proj.weight"): TensorSpec((h, i))}
+
+    def bind(self, tensors) -> None:
+        self.up, self.down = tensors[self.names["up"]], tensors[self.names["down"]]
+
+    def forward(self, x, residual):
+        ops = self.rt.ops
+        m = ops.activate(ops.linear(x, self.up, out_dtype=torch.float32), self.activation, self.rt.dtype)
+        return ops.linear(m, self.down, accumulate_into=residual, defer=True)
+
+    def parameters_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.up, self.down))
+
+    def flops(self, rows) -> int:
+        return 2 * sum(n for n, _ in rows) * 2 * self.hidden * self.inter

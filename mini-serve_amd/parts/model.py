@@ -81,7 +81,8 @@ class DecoderModel:
             weights[name] = weights[source]  # the same tensor under its second name
 
         def local(prefix: str, part_type, part_spec) -> dict:
-            names = list(part_type.tensors(part_spec)) + list(part_type.aliases(part_spec))
+            declared = part_type.tensors(part_spec)
+            names = [n for n, ts in declared.items() if not ts.optional] + list(part_type.aliases(part_spec))
             return {n: weights[prefix + n] for n in names}
 
         self.embedding = part_class("embedding", spec.embedding)(spec.embedding, rt)
@@ -103,7 +104,9 @@ class DecoderModel:
     # ------------------------------------------------------------------ cache needs
 
     def cache_slots(self) -> list[CacheSlotNeed]:
-        """One entry per cache slot of the run order, from the mixer that writes it."""
+        """One entry per cache slot of the run order, from the mixer that writes it. An entry that reads a slot
+        another entry wrote must keep the same planes and state; its window may differ, and the slot then keeps
+        the widest of them (every token, if one of its readers sees every token)."""
         needs: dict[int, CacheSlotNeed] = {}
         for e in self.spec.run_order:
             if e.cache is None:
@@ -112,10 +115,17 @@ class DecoderModel:
             need = CacheSlotNeed(e.cache, mixer.kv_need(), mixer.state_need())
             if e.writes_cache:
                 needs[e.cache] = need
-            elif (needs[e.cache].kv, needs[e.cache].state) != (need.kv, need.state):
+                continue
+            held = needs[e.cache]
+            same = (held.kv is None) == (need.kv is None) and (held.kv is None or held.kv.planes == need.kv.planes)
+            if not same or held.state != need.state:
                 raise ValueError(
-                    f"layer {e.layer} reads cache slot {e.cache} but needs {need}, the slot holds {needs[e.cache]}"
+                    f"layer {e.layer} reads cache slot {e.cache} but needs {need}, the slot holds {held}"
                 )
+            if held.kv is not None and (held.kv.window, held.kv.keep_first) != (need.kv.window, need.kv.keep_first):
+                window = 0 if 0 in (held.kv.window, need.kv.window) else max(held.kv.window, need.kv.window)
+                keep = max(held.kv.keep_first, need.kv.keep_first) if window else 0
+                needs[e.cache] = CacheSlotNeed(e.cache, KVNeed(held.kv.planes, window, keep), held.state)
         return [needs[s] for s in sorted(needs)]
 
     # ------------------------------------------------------------------ forward

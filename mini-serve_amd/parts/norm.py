@@ -1,9 +1,14 @@
 """RMSNorm: ``y = w * x * rsqrt(mean(x^2) + eps)``, statistics and scaling in float32, plain weight
 (not ``1 + w``) as in the reference (miniserve/model/qwen3.py:78-82). The reference rounds to the
 model dtype before the weight product; here the whole expression is evaluated in float32 and
-rounded once, which is what its fused operators do (miniserve/model/fused.py:188-194)."""
+rounded once, which is what its fused operators do (miniserve/model/fused.py:188-194).
+
+``offset`` (optional, no counterpart in the reference): the stored weight lies around zero and the norm multiplies by
+``offset + w`` (``offset = 1``: the "one plus weight" form). The sum is formed once, in float32, when the weight is bound."""
 
 from __future__ import annotations
+
+import torch
 
 from ..config.spec import PartSpec
 from .base import Norm, TensorSpec
@@ -16,20 +21,27 @@ class RMSNorm(Norm):
         super().__init__(spec, rt)
         self.width = int(spec["width"])
         self.eps = float(spec["eps"])
+        self.offset = float(spec.get("offset") or 0.0)
         self.weight = None
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
-        return {spec["tensor"]: TensorSpec((int(spec["width"]),), init="ones")}
+        # a weight stored around zero is drawn around zero
+        return {spec["tensor"]: TensorSpec((int(spec["width"]),), init="uniform" if spec.get("offset") else "ones")}
 
     def bind(self, tensors) -> None:
         self.weight = tensors[self.spec["tensor"]]
+        if self.offset:
+            self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
 
     def forward(self, x, rows=None, add=None):
         """``x``: float32 ``[T, width]``; ``rows``: optional int32 row indices to normalise (the
         others are skipped); ``add``: a pending sum added into the normalised rows of ``x`` first.
         Returns the compute dtype, ``[T or len(rows), width]``."""
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows, add)
+
+    def add_normed(self, residual, stream) -> None:
+        self.rt.ops.normed_mean_add(residual, [stream], [self.weight], self.eps, 1.0)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

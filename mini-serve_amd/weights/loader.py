@@ -92,7 +92,7 @@ def load_weights(
                     weights[name] = _place(sf.get_tensor(name), ts.kind, dtype).to(device).contiguous()
                 except TypeError as e:
                     mismatched.append(f"{name}: {e}")
-    missing = sorted(want.keys() - weights.keys() - {m.split(":")[0] for m in mismatched})
+    missing = sorted({n for n, ts in want.items() if not ts.optional} - weights.keys() - {m.split(":")[0] for m in mismatched})
     if missing or unexpected or mismatched:
         raise WeightsError(path, missing, sorted(unexpected), sorted(mismatched))
     for name, source in aliases.items():

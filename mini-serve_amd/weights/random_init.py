@@ -45,6 +45,8 @@ def random_tensors(
     f32 = dict(dtype=torch.float32, device=device)
     out = {}
     for name, ts in sorted(expected_tensors(spec).items()):
+        if ts.optional:
+            continue
         if ts.kind == "int":
             out[name] = torch.randint(0, ts.high, ts.shape, generator=gen, dtype=torch.int32, device=device)
             continue
