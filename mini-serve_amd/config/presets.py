@@ -1,5 +1,5 @@
 """Named ``config.json`` dictionaries: two tiny shapes that differ in every size and option, one
-tiny windowed shape, the three benchmark shapes, and one tiny Kakunex model (random weights; no checkpoint is fetched).
+tiny windowed shape, the three benchmark shapes, one tiny Kakunex and one tiny Fimolix model (random weights; no checkpoint is fetched).
 
 The reference names models by size and maps them to pinned downloads
 (miniserve/model/weights.py:24-29); without a network the names map to shapes instead.
@@ -86,6 +86,34 @@ def _kakunex_tiny() -> dict:
 
 
 PRESETS["kakunex-tiny"] = _kakunex_tiny()
+
+
+def _fimolix_tiny() -> dict:
+    """Four layers that hold every part of the architecture once: a latent attention with a window, a differential
+    attention with a convolution of three taps, a second latent attention that reads the first one's cache through a
+    wider window and has no feed-forward, and a differential attention whose heads share one key/value head."""
+    rot = {"base": 5000.0, "dims": 8}
+
+    def latent(heads, dim, vdim, size, ff, kv_from=None):
+        m = {"heads": heads, "dim": dim, "rot_dim": 8, "vdim": vdim, "kv_rank": 40, "scale": (dim + 8) ** -0.5, "rot": rot,
+             "mask": {"size": size}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+    def attention(heads, kv_heads, dim, vdim, conv, diff, ff):
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "softcap": 20.0, "conv": conv,
+             "diff": diff}
+        return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+    return {
+        "architecture": "Fimolix", "vocab": 311, "width": 96, "norm": {"eps": 1e-5},
+        "layers": [latent(4, 16, 24, 24, 160), attention(4, 2, 16, 32, 3, 0.4, 128), latent(2, 24, 16, 56, None, kv_from=0),
+                   attention(3, 1, 32, 16, 4, 0.6, 160)],
+    }
+
+
+PRESETS["fimolix-tiny"] = _fimolix_tiny()
 
 
 def preset(name: str) -> dict:

@@ -21,7 +21,8 @@
 //   value_share     this many consecutive key heads read the same value head (key head i: value head i / value_share;
 //                   the value cache then has Hkv / value_share heads): several score maps over one set of values;
 //   values_in_keys  the values are the first Dv elements of the key rows themselves (one vector per token serves as
-//                   key and as value); no value cache is read.
+//                   key and as value); no value cache is read;
+//   out_f32         the result is written as float32 whatever the storage type (for a consumer that norms it).
 // Head sizes up to 256, or, with at most eight waves, up to 1024.
 #include "common.h"
 
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
     const int* __restrict__ block_table, int table_width, const int* __restrict__ token_list,
     const int* __restrict__ token_row, const int* __restrict__ pos, T* __restrict__ out, int Hq, int Hkv, int D, int Dv,
     int page_size, float scale, int window, int keep_first, float softcap, const float* __restrict__ sinks, int value_share,
-    int values_in_keys) {
+    int values_in_keys, float* __restrict__ out32) {
   __shared__ __attribute__((aligned(16))) float qs[MAXD];
   __shared__ float ps[NW][WAVE];
   __shared__ float ml[NW][2];
@@ -204,10 +205,13 @@ __global__ __launch_bounds__(NW * WAVE) void paged_attention_generic_kernel(
     const float c = expf(m_run - m_all);
     inv = c / (l_run * c + expf(sink - m_all));
   }
+  float* ov32 = out32 ? out32 + ((size_t)t * Hq + h) * Dv : nullptr;  // the result unrounded, whatever the storage
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = lane + i * WAVE;
-    if (e < Dv) ov[e] = from_f32<T>(o[i] * inv);
+    if (e >= Dv) continue;
+    if (ov32) ov32[e] = o[i] * inv;
+    else ov[e] = from_f32<T>(o[i] * inv);
   }
 }
 
@@ -216,7 +220,7 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
                                           const int* token_row, const int* pos, void* out, int tokens, int Hq, int Hkv,
                                           int D, int Dv, int page_size, float scale, int window, int keep_first, int waves,
                                           float softcap, const float* sinks, int value_share, int values_in_keys,
-                                          hipStream_t st) {
+                                          int out_f32, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (D <= 0 || D > MAX_WIDE_HEAD_DIM || Dv <= 0 || Dv > MAX_WIDE_HEAD_DIM || Hq <= 0 || Hkv <= 0 || Hq % Hkv || page_size <= 0 ||
       window < 0 || keep_first < 0 || table_width <= 0 || Hq > 65535 || q_stride < Hq * D || (waves != 1 && waves != 8 && waves != 16) ||
@@ -230,7 +234,7 @@ extern "C" int ms_paged_attention_generic(const void* q, int q_stride, const voi
 #define GA(T, NW, MAXD)                                                                                                      \
   paged_attention_generic_kernel<T, NW, MAXD><<<grid, NW * WAVE, 0, st>>>(                                                   \
       (const T*)q, q_stride, (const T*)kc, (const T*)vc, block_table, table_width, token_list, token_row, pos, (T*)out, Hq, Hkv, D, \
-      Dv, page_size, scale, window, keep_first, softcap, sinks, value_share, values_in_keys)
+      Dv, page_size, scale, window, keep_first, softcap, sinks, value_share, values_in_keys, out_f32 ? (float*)out : nullptr)
   if (wide) {
     if (is_bf16) {
       if (waves == 8) GA(bf16, 8, MAX_WIDE_HEAD_DIM); else GA(bf16, 1, MAX_WIDE_HEAD_DIM);

@@ -115,10 +115,10 @@ extern "C" int ms_conv_norm_store(const float* x, int ld, const void* cw, int w_
 // ---------------------------------------------------------------------------------------------
 // Two score maps over the same values, combined per head: o = a1 - lambda * a2, divided by its root mean square over
 // the head's E values (eps inside the root, no weight), times out_scale. `a` holds the maps' outputs as the attention
-// kernel leaves them, [tokens, G, 2, R, E]: key/value group, map, the group's R query heads. Output [tokens, G * R * E],
+// kernel leaves them (float32, or the storage type), [tokens, G, 2, R, E]: key/value group, map, the group's R query heads. Output [tokens, G * R * E],
 // head h = g * R + r. One block per token, a wave per head in turn.
-template <typename T>
-__global__ __launch_bounds__(256) void map_difference_norm_kernel(const T* __restrict__ a, T* __restrict__ out, int G, int R, int E,
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void map_difference_norm_kernel(const T* __restrict__ a, TO* __restrict__ out, int G, int R, int E,
                                                                   float lambda, float eps, float out_scale) {
   const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const T* row = a + (size_t)t * G * 2 * R * E;
@@ -132,17 +132,18 @@ __global__ __launch_bounds__(256) void map_difference_norm_kernel(const T* __res
       ss += o * o;
     }
     const float k = out_scale / sqrtf(wave_sum(ss) / (float)E + eps);
-    T* dst = out + ((size_t)t * G * R + h) * E;
-    for (int e = lane; e < E; e += WAVE) dst[e] = from_f32<T>((to_f32(a1[e]) - lambda * to_f32(a2[e])) * k);
+    TO* dst = out + ((size_t)t * G * R + h) * E;
+    for (int e = lane; e < E; e += WAVE) dst[e] = from_f32<TO>((to_f32(a1[e]) - lambda * to_f32(a2[e])) * k);
   }
 }
 
-extern "C" int ms_map_difference_norm(const void* a, void* out, int is_bf16, int tokens, int G, int R, int E, float lambda,
-                                      float eps, float out_scale, hipStream_t st) {
+extern "C" int ms_map_difference_norm(const void* a, void* out, int in_is_bf16, int out_is_bf16, int tokens, int G, int R, int E,
+                                      float lambda, float eps, float out_scale, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (G <= 0 || R <= 0 || E <= 0 || !(eps >= 0.f)) return MS_BAD_ARG;
-  if (is_bf16) map_difference_norm_kernel<bf16><<<tokens, 256, 0, st>>>((const bf16*)a, (bf16*)out, G, R, E, lambda, eps, out_scale);
-  else map_difference_norm_kernel<float><<<tokens, 256, 0, st>>>((const float*)a, (float*)out, G, R, E, lambda, eps, out_scale);
+  if (G <= 0 || R <= 0 || E <= 0 || !(eps >= 0.f) || (in_is_bf16 && !out_is_bf16)) return MS_BAD_ARG;
+  if (in_is_bf16) map_difference_norm_kernel<bf16, bf16><<<tokens, 256, 0, st>>>((const bf16*)a, (bf16*)out, G, R, E, lambda, eps, out_scale);
+  else if (out_is_bf16) map_difference_norm_kernel<float, bf16><<<tokens, 256, 0, st>>>((const float*)a, (bf16*)out, G, R, E, lambda, eps, out_scale);
+  else map_difference_norm_kernel<float, float><<<tokens, 256, 0, st>>>((const float*)a, (float*)out, G, R, E, lambda, eps, out_scale);
   return launch_status();
 }
 

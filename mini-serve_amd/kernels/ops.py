@@ -56,11 +56,11 @@ _SIGNATURES = {
     "ms_splitk_reduce": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void,
                                    _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int,
-                                   _c_float, _c_void, _c_int, _c_int, _c_void],
+                                   _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_conv_norm_store": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                            _c_void, _c_float, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                            _c_int, _c_int, _c_int, _c_void],
-    "ms_map_difference_norm": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void],
+    "ms_map_difference_norm": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void],
     "ms_latent_prepare": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_int, _c_float, _c_void, _c_void,
                           _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -665,7 +665,8 @@ def decode_attention_fused(qkv, q_weight, k_weight, eps, rope, store, k_cache, v
 
 def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv_heads, head_dim, scale, window,
                     value_dim: int | None = None, keep_first: int = 0, exact_weights: bool = False, softcap: float = 0.0,
-                    sinks: torch.Tensor | None = None, value_share: int = 1, values_in_keys: bool = False):
+                    sinks: torch.Tensor | None = None, value_share: int = 1, values_in_keys: bool = False,
+                    out_dtype=None):
     """Attention of the batch's new tokens over the cache. ``qkv [T, >= Hq D]`` holds the queries
     in its first ``Hq * D`` columns. Returns ``[T, Hq * Dv]`` (``Dv = D`` unless ``value_dim`` is given).
     A query at position p sees keys ``max(0, p - window + 1) .. p`` (``window == 0``: all up to p) and, with a
@@ -680,11 +681,15 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     ``softcap > 0`` bounds a scaled score ``s`` to ``softcap * tanh(s / softcap)``; ``sinks`` (float32 ``[Hq]``) adds
     ``exp(sinks[h])`` to head ``h``'s softmax denominator; ``value_share = n`` lets ``n`` consecutive key heads weigh
     the same value head (``v_cache`` then has ``Hkv / n`` heads); ``values_in_keys`` takes the first ``Dv`` elements
-    of each key row as that token's value (``v_cache`` is None)."""
+    of each key row as that token's value (``v_cache`` is None); ``out_dtype=torch.float32`` returns the result
+    unrounded whatever the cache's dtype."""
     _dev(qkv, "qkv", (F32, BF16), 2)
     t = qkv.shape[0]
     dv = head_dim if value_dim is None else int(value_dim)
-    special = bool(softcap) or sinks is not None or value_share != 1 or values_in_keys
+    out_f32 = out_dtype == F32 and qkv.dtype != F32
+    if out_dtype not in (None, F32, qkv.dtype):
+        raise TypeError(f"the result comes in the queries' dtype or in float32, not {out_dtype}")
+    special = bool(softcap) or sinks is not None or value_share != 1 or values_in_keys or out_f32
     if special:
         page = _check_special_caches(k_cache, v_cache, qkv.dtype, num_kv_heads, head_dim, dv, value_share, values_in_keys)
         if sinks is not None:
@@ -711,7 +716,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     _dev(batch.positions, "positions", I32, 1)
     if batch.token_row.shape[0] != t or batch.positions.shape[0] != t or block_table.shape[0] < batch.num_rows:
         raise ValueError("batch metadata does not match the number of tokens or rows")
-    out = torch.empty((t, num_heads * dv), dtype=qkv.dtype, device=qkv.device)
+    out = torch.empty((t, num_heads * dv), dtype=F32 if out_f32 else qkv.dtype, device=qkv.device)
     lib = library()
     common = (block_table.data_ptr(), block_table.shape[1])
     meta = (batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr())
@@ -721,7 +726,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     if not fast:
         generic = (qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), _ptr(v_cache), int(qkv.dtype == BF16), *common)
         shape = (num_heads, num_kv_heads, head_dim, dv, page, float(scale), int(window), int(keep_first))
-        extra = (float(softcap), _ptr(sinks), int(value_share), int(values_in_keys))
+        extra = (float(softcap), _ptr(sinks), int(value_share), int(values_in_keys), int(out_f32))
         tile_tokens = 0 if special else lib.ms_paged_attention_tiled_tokens(num_heads // num_kv_heads, head_dim, dv)
         lens = getattr(batch, "row_lens", None)
         if special and lens is not None and 0 < n_dec < t:
@@ -1084,16 +1089,21 @@ def conv_norm_store(x, conv_weight, taps: int, state, batch, q_weight, k_weight,
 
 
 def map_difference_norm(a: torch.Tensor, groups: int, per_group: int, value_dim: int, weight: float, eps: float,
-                        out_scale: float) -> torch.Tensor:
+                        out_scale: float, out_dtype=None) -> torch.Tensor:
     """``a [T, groups * 2 * per_group * Dv]`` holds two attention maps' outputs per head, ordered (group, map, head of
     the group). Per head: ``o = a1 - weight * a2``, divided by its root mean square over ``Dv`` (``eps`` inside the
-    root), times ``out_scale``. Returns ``[T, groups * per_group * Dv]`` in ``a``'s dtype, float32 arithmetic."""
+    root), times ``out_scale``. Returns ``[T, groups * per_group * Dv]`` in ``out_dtype`` (default: ``a``'s), float32
+    arithmetic. The difference of two close maps loses what their rounding lost: give ``a`` in float32."""
     _dev(a, "a", (F32, BF16), 2)
     if a.shape[1] != groups * 2 * per_group * value_dim:
         raise ValueError(f"a has width {a.shape[1]}, expected {groups * 2 * per_group * value_dim}")
-    out = torch.empty((a.shape[0], groups * per_group * value_dim), dtype=a.dtype, device=a.device)
-    _check(library().ms_map_difference_norm(a.data_ptr(), out.data_ptr(), int(a.dtype == BF16), a.shape[0], groups, per_group,
-                                            value_dim, float(weight), float(eps), float(out_scale), _stream()), "map_difference_norm")
+    out_dtype = a.dtype if out_dtype is None else out_dtype
+    if out_dtype not in (F32, BF16) or (a.dtype == BF16 and out_dtype != BF16):
+        raise TypeError(f"unsupported dtypes {a.dtype} -> {out_dtype}")
+    out = torch.empty((a.shape[0], groups * per_group * value_dim), dtype=out_dtype, device=a.device)
+    _check(library().ms_map_difference_norm(a.data_ptr(), out.data_ptr(), int(a.dtype == BF16), int(out_dtype == BF16), a.shape[0],
+                                            groups, per_group, value_dim, float(weight), float(eps), float(out_scale), _stream()),
+           "map_difference_norm")
     return out
 
 

@@ -129,8 +129,9 @@ class DifferentialAttention(Mixer):
                                 eps, cache.slots, cache.k, cache.v, 2 * self.heads, 2 * self.kv_heads, self.kv_heads, self.head_dim,
                                 self.value_dim, self.rt.dtype)
         a = ops.paged_attention(q, cache.k, cache.v, cache.block_table, batch, 2 * self.heads, 2 * self.kv_heads, self.head_dim,
-                                self.scale, 0, self.value_dim, softcap=self.softcap, value_share=2)
-        o = ops.map_difference_norm(a, self.kv_heads, self.group, self.value_dim, self.lam, self.eps, 1.0 - self.lambda_offset)
+                                self.scale, 0, self.value_dim, softcap=self.softcap, value_share=2, out_dtype=torch.float32)
+        o = ops.map_difference_norm(a, self.kv_heads, self.group, self.value_dim, self.lam, self.eps, 1.0 - self.lambda_offset,
+                                    self.rt.dtype)
         return ops.linear(o, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:

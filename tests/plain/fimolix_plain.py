@@ -114,7 +114,7 @@ def differential_attention(h, w, m, eps):
     q = rms_norm(q, w["q.norm"], eps)
     k = rms_norm(k, w["k.norm"], eps)
     lam = math.exp(float((w["lq1"] * w["lk1"]).sum())) - math.exp(float((w["lq2"] * w["lk2"]).sum())) + m["diff"]
-    cap = m["softcap"]
+    cap = m.get("softcap")  # absent: the scores are not capped
     seen = causal(T)
     out = np.zeros((T, H, E))
     for head in range(H):
@@ -122,7 +122,8 @@ def differential_attention(h, w, m, eps):
         maps = []
         for which in range(2):
             s = (q[:, head, which] @ k[:, g, which].T) * m["scale"]
-            s = cap * np.tanh(s / cap)
+            if cap:
+                s = cap * np.tanh(s / cap)
             maps.append(masked_softmax(s, seen) @ v[:, g])
         o = maps[0] - lam * maps[1]
         out[:, head] = unit_rms(o, eps) * (1.0 - m["diff"])
@@ -149,7 +150,7 @@ def latent_attention(h, w, m, eps, positions, kept):
     k_plain = (c @ w["uk"].T).reshape(T, H, D)
     v = (c @ w["uv"].T).reshape(T, H, E)
     gate = sigmoid(h @ w["g"].T)  # [T, H]
-    seen = sliding(T, m["mask"]["size"])
+    seen = sliding(T, m["mask"]["size"]) if m.get("mask") else causal(T)  # absent: every earlier token is seen
     out = np.zeros((T, H, E))
     for head in range(H):
         s = (q_plain[:, head] @ k_plain[:, head].T + q_turned[:, head] @ kr.T) * m["scale"]
@@ -194,3 +195,11 @@ def forward(cfg, weights, tokens, return_layers=False):
         after.append(x.copy())
     logits = one_plus_norm(x, weights["final.norm"], eps) @ weights["embed"].T
     return (logits, np.stack(after)) if return_layers else logits
+
+
+def greedy(cfg, weights, prompt, new_tokens):
+    """The ``new_tokens`` tokens that greedy decoding appends to ``prompt`` (the whole sequence is run again each time)."""
+    toks = list(prompt)
+    for _ in range(new_tokens):
+        toks.append(int(np.argmax(forward(cfg, weights, toks)[-1])))
+    return toks[len(prompt):]
