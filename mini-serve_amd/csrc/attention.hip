@@ -682,6 +682,209 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_kernel(
   }
 }
 
+// tanh on the hardware's exp2 and reciprocal: 1 - 2 / (1 + e^(2x)), about one unit in the last place of float32 near
+// zero and exact at the ends (e^(2x) = inf gives 1, 0 gives -1).
+__device__ __forceinline__ float tanh_fast(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * 2.885390081777927f));
+}
+
+// The same kernel for heads of any size that is a multiple of 32 (keys) and 16 (values), and for the options of the
+// generic form: a soft cap on the scores, a sink per query head, key heads that share a value head, float32 results.
+// What differs: the key size D is a run-time number, and the query fragments are fetched again for every key tile (from
+// the cache: a block's 64 query rows are what all its tiles share) instead of living in registers; a block owns DVC of a
+// head's Dv value elements (blockIdx.z names the run), so a head of 512 values is four blocks that each form the scores
+// again. The keys' loads are issued per run of 64 elements, two runs under way.
+template <int DVC>
+__global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+    const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
+    const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
+    float* __restrict__ out32, int Hq, int Hkv, int D, int Dv, float scale, int window, int keep_first, float softcap,
+    const float* __restrict__ sinks, int value_share) {
+  constexpr int PS = WAVE + 4;  // floats between a wave's rows of weights
+  __shared__ __attribute__((aligned(16))) float Pw[4][16][PS];
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
+  const int kvh = blockIdx.y, g = Hq / Hkv, e0 = blockIdx.z * DVC;
+  const int Hv = Hkv / value_share, vh = kvh / value_share;
+  const int first = tile_first[blockIdx.x], count = tile_count[blockIdx.x], rows = count * g;
+  const int* table = block_table + (size_t)token_row[first] * table_width;
+  const int p_first = pos[first], p_last = p_first + count - 1;
+  const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  const int kept = keep_first < lo_first ? keep_first : lo_first;
+  const int chunks = D / 32;
+
+  // this lane's query row as the A operand: row 16 wave + l16, elements 32 kk + 8 grp .. + 7
+  const int qr = wave * 16 + l16;
+  const bf16* qp = qr < rows ? q + (size_t)(first + qr / g) * q_stride + (size_t)(kvh * g + qr % g) * D + grp * 8 : nullptr;
+  int pr[4], lor[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + grp * 4 + r;
+    pr[r] = row < rows ? p_first + row / g : -1;
+    lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
+  }
+  float m_run[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
+  floatx4 o[DVC / 16], l_run = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int et = 0; et < DVC / 16; ++et) o[et] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 ones;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) ones[u] = static_cast<bf16>(1.f);
+  const float cap_in = softcap > 0.f ? scale / softcap : 0.f;
+
+  const int kept_tiles = (kept + WAVE - 1) / WAVE;
+  const int first_window_tile = lo_first / WAVE > kept_tiles ? lo_first / WAVE : kept_tiles;
+  const int tiles = kept_tiles + (p_last / WAVE - first_window_tile + 1);
+  for (int ti = 0; ti < tiles; ++ti) {
+    const int j0 = (ti < kept_tiles ? ti : first_window_tile + (ti - kept_tiles)) * WAVE;
+    const int4 pg4 = *reinterpret_cast<const int4*>(table + j0 / MFMA_PAGE);
+    const int pages[4] = {pg4.x, pg4.y, pg4.z, pg4.w};
+    bf16x8 vf[2][DVC / 16];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int jb = j0 + ks * 32 + grp * 8;  // this lane's 8 keys as the B operand: one run of a page
+      const int page = pages[ks * 2 + grp / 2];
+      const bool seen = jb <= p_last && (jb + 8 > lo_first || jb < kept) && page >= 0;
+      const bf16* vp = vc + (((size_t)(seen ? page : 0) * Hv + vh) * Dv + e0) * MFMA_PAGE + (jb % MFMA_PAGE);
+#pragma unroll
+      for (int et = 0; et < DVC / 16; ++et) vf[ks][et] = seen ? load_bf16x8(vp + (size_t)(et * 16 + l16) * MFMA_PAGE) : zero_bf16x8();
+    }
+    const bf16* kp[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
+      const bool seen = j <= p_last && (j >= lo_first || j < kept) && pages[t] >= 0;
+      kp[t] = seen ? kc + (((size_t)pages[t] * Hkv + kvh) * MFMA_PAGE + l16) * D + grp * 8 : nullptr;
+    }
+    floatx4 s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int kk = 0; kk < chunks; kk += 2) {
+      bf16x8 qf[2], kf[2][4];
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const bool in = kk + c < chunks;
+        qf[c] = (in && qp) ? load_bf16x8(qp + (kk + c) * 32) : zero_bf16x8();
+#pragma unroll
+        for (int t = 0; t < 4; ++t) kf[c][t] = (in && kp[t]) ? load_bf16x8(kp[t] + (kk + c) * 32) : zero_bf16x8();
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], kf[c][t], s[t], 0, 0, 0);
+    }
+    float corr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float mx = -INFINITY;
+      bool ok[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int j = j0 + t * 16 + l16;
+        ok[t] = j <= pr[r] && (j >= lor[r] || j < keep_first);
+        const float sc = softcap > 0.f ? softcap * tanh_fast(s[t][r] * cap_in) : s[t][r] * scale;
+        s[t][r] = ok[t] ? sc : -INFINITY;
+        mx = fmaxf(mx, s[t][r]);
+      }
+      mx = row16_max(mx);
+      const float m_new = fmaxf(m_run[r], mx);
+      const bool none = m_new == -INFINITY;  // no key of this row so far
+      corr[r] = none ? 1.f : exp_fast(m_run[r] - m_new);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) Pw[wave][grp * 4 + r][t * 16 + l16] = (ok[t] && !none) ? exp_fast(s[t][r] - m_new) : 0.f;
+      l_run[r] *= corr[r];
+      m_run[r] = m_new;
+    }
+#pragma unroll
+    for (int et = 0; et < DVC / 16; ++et)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[et][r] *= corr[r];
+    __builtin_amdgcn_wave_barrier();  // a wave's own rows: its order of LDS operations is enough
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const float4 a0 = *reinterpret_cast<const float4*>(&Pw[wave][l16][ks * 32 + grp * 8]);
+      const float4 a1 = *reinterpret_cast<const float4*>(&Pw[wave][l16][ks * 32 + grp * 8 + 4]);
+      const float pv[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+      bf16x8 hi, mid, low;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const bf16 h = static_cast<bf16>(pv[u]);
+        const float r1 = pv[u] - static_cast<float>(h);
+        const bf16 m = static_cast<bf16>(r1);
+        hi[u] = h;
+        mid[u] = m;
+        low[u] = static_cast<bf16>(r1 - static_cast<float>(m));
+      }
+#pragma unroll
+      for (int et = 0; et < DVC / 16; ++et) {
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, vf[ks][et], o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, vf[ks][et], o[et], 0, 0, 0);
+        o[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, vf[ks][et], o[et], 0, 0, 0);
+      }
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, ones, l_run, 0, 0, 0);
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mid, ones, l_run, 0, 0, 0);
+      l_run = __builtin_amdgcn_mfma_f32_16x16x32_bf16(low, ones, l_run, 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();  // the weights have been read before the next tile's are written
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + grp * 4 + r;
+    if (row >= rows) continue;
+    const int head = kvh * g + row % g;
+    float inv = 1.f / l_run[r];
+    if (sinks) {  // exp(sink) joins the denominator: both are brought to the larger of the two maxima first
+      const float sink = sinks[head], m_all = fmaxf(m_run[r], sink);
+      const float c = expf(m_run[r] - m_all);
+      inv = c / (l_run[r] * c + expf(sink - m_all));
+    }
+    const size_t at = ((size_t)(first + row / g) * Hq + head) * Dv + e0;
+#pragma unroll
+    for (int et = 0; et < DVC / 16; ++et) {
+      if (out32) out32[at + et * 16 + l16] = o[et][r] * inv;
+      else out[at + et * 16 + l16] = static_cast<bf16>(o[et][r] * inv);
+    }
+  }
+}
+
+// The run of value elements a block of the wide form owns (0: it does not take the shape): keys a multiple of 32,
+// values a multiple of 16, up to 64 query heads per key head, 16-token pages.
+extern "C" int ms_paged_attention_tiled_mfma_wide_chunk(int group, int D, int Dv, int page_size) {
+  if (page_size != MFMA_PAGE || group < 1 || group > TILED_ROWS || D < 32 || D % 32 || Dv < 16 || Dv % 16) return 0;
+  return Dv % 128 == 0 ? 128 : Dv % 64 == 0 ? 64 : Dv % 32 == 0 ? 32 : 16;
+}
+
+// As ms_paged_attention_tiled_mfma, with the generic form's options; tiles of TILED_ROWS / group tokens. out_f32: the
+// result is float32.
+extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, const void* kc, const void* vc,
+                                                  const int* block_table, int table_width, const int* tile_first,
+                                                  const int* tile_count, int tiles, const int* token_row, const int* pos, void* out,
+                                                  int out_f32, int Hq, int Hkv, int D, int Dv, int page_size, float scale, int window,
+                                                  int keep_first, float softcap, const float* sinks, int value_share, hipStream_t st) {
+  if (tiles <= 0) return MS_OK;
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || window < 0 || keep_first < 0 || table_width <= 0 || table_width % 4 || Hkv > 65535 ||
+      q_stride < Hq * D || q_stride % 8 || tile_first == nullptr || tile_count == nullptr || !(softcap >= 0.f) || value_share < 1 ||
+      Hkv % value_share)
+    return MS_BAD_ARG;
+  const int chunk = ms_paged_attention_tiled_mfma_wide_chunk(Hq / Hkv, D, Dv, page_size);
+  if (chunk == 0 || Dv / chunk > 65535) return MS_UNSUPPORTED;
+  if (window == 0) keep_first = 0;
+  dim3 grid(tiles, Hkv, Dv / chunk);
+#define TW(CC)                                                                                                                 \
+  paged_attention_tiled_mfma_wide_kernel<CC><<<grid, 256, 0, st>>>(                                                            \
+      (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, pos, \
+      out_f32 ? nullptr : (bf16*)out, out_f32 ? (float*)out : nullptr, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks,   \
+      value_share)
+  if (chunk == 128) TW(128);
+  else if (chunk == 64) TW(64);
+  else if (chunk == 32) TW(32);
+  else TW(16);
+#undef TW
+  return launch_status();
+}
+
 // 1 where the matrix-core form of the tiled kernel takes the shape (bfloat16 storage).
 extern "C" int ms_paged_attention_tiled_mfma_ok(int D, int Dv, int page_size) {
   return page_size == MFMA_PAGE && (D == 32 || D == 64 || D == 96 || D == 128) && (Dv == 16 || Dv == 32 || Dv == 64 || Dv == 128);

@@ -155,14 +155,17 @@ extern "C" int ms_map_difference_norm(const void* a, void* out, int in_is_bf16, 
 //   and sine are rope[t][j] and rope[t][rot/2 + j]; the rest pass.
 //   q_plain [tokens, H * Dn]: the plain query parts (a per-head matrix product takes them into the latent's space);
 //   q_full [tokens, H * (C + R)]: only the turned parts are written here, behind each head's C columns;
-//   cache row of the token's slot, [C + R]: the latent after its RMS norm (weight cw), then the turned key part.
+//   cache row of the token's slot, [C + R]: the latent after its RMS norm (weight cw), then the turned key part;
+//   the normed latent once more as the token's value, transposed within the page ([pages, C, page_size]): the tokens of
+//   one element side by side, the order in which the matrix cores take the values.
 // One block per token.
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __restrict__ x, int ld, int q_col, int kv_col,
                                                              const float* __restrict__ rope, int rot, int pairing,
                                                              const TW* __restrict__ cw, float eps, T* __restrict__ q_plain,
                                                              T* __restrict__ q_full, const int* __restrict__ slots,
-                                                             T* __restrict__ kc, int H, int Dn, int R, int C) {
+                                                             T* __restrict__ kc, T* __restrict__ vc, int page_size, int H, int Dn,
+                                                             int R, int C) {
   __shared__ float red[256 / WAVE];
   const int t = blockIdx.x;
   const float* row = x + (size_t)t * ld;
@@ -192,22 +195,30 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __rest
   float ss = 0.f;
   for (int j = threadIdx.x; j < C; j += 256) ss += kv[j] * kv[j];
   const float r = 1.f / sqrtf(block_sum<256>(ss, red) / (float)C + eps);
-  T* dst = kc + (size_t)slots[t] * (C + R);
-  for (int j = threadIdx.x; j < C; j += 256) dst[j] = from_f32<T>(kv[j] * r * to_f32(cw[j]));
+  const int slot = slots[t], page = slot / page_size, off = slot % page_size;
+  T* dst = kc + (size_t)slot * (C + R);
+  T* val = vc + (size_t)page * C * page_size + off;
+  for (int j = threadIdx.x; j < C; j += 256) {
+    const T c = from_f32<T>(kv[j] * r * to_f32(cw[j]));
+    dst[j] = c;
+    val[(size_t)j * page_size] = c;
+  }
   for (int j = threadIdx.x; j < R; j += 256) dst[C + j] = from_f32<T>(turned(kv + C, j));
 }
 
 extern "C" int ms_latent_prepare(const float* x, int ld, int q_col, int kv_col, const float* rope, int rot, int pairing,
                                  const void* cw, int w_is_bf16, float eps, void* q_plain, void* q_full, const int* slots,
-                                 void* kc, int out_is_bf16, int tokens, int H, int Dn, int R, int C, hipStream_t st) {
+                                 void* kc, void* vc, int page_size, int out_is_bf16, int tokens, int H, int Dn, int R, int C,
+                                 hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (H <= 0 || Dn <= 0 || R < 0 || C <= 0 || rot < 0 || rot > R || rot % 2 || (rot > 0 && rope == nullptr) ||
       (pairing != MS_ROPE_HALVES && pairing != MS_ROPE_ADJACENT) || q_col < 0 || ld < q_col + H * (Dn + R) ||
-      (kv_col >= 0 && (ld < kv_col + C + R || slots == nullptr || kc == nullptr || cw == nullptr)) || !(eps >= 0.f))
+      (kv_col >= 0 && (ld < kv_col + C + R || slots == nullptr || kc == nullptr || vc == nullptr || cw == nullptr || page_size < 1)) ||
+      !(eps >= 0.f))
     return MS_BAD_ARG;
 #define LP(T, TW)                                                                                                             \
   latent_prepare_kernel<T, TW><<<tokens, 256, 0, st>>>(x, ld, q_col, kv_col, rope, rot, pairing, (const TW*)cw, eps, (T*)q_plain, \
-                                                       (T*)q_full, slots, (T*)kc, H, Dn, R, C)
+                                                       (T*)q_full, slots, (T*)kc, (T*)vc, page_size, H, Dn, R, C)
   if (out_is_bf16) {
     if (w_is_bf16) LP(bf16, bf16); else LP(bf16, float);
   } else {

@@ -62,7 +62,11 @@ _SIGNATURES = {
                            _c_int, _c_int, _c_int, _c_void],
     "ms_map_difference_norm": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_void],
     "ms_latent_prepare": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_int, _c_float, _c_void, _c_void,
-                          _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+                          _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_paged_attention_tiled_mfma_wide": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
+                                           _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
+                                           _c_void, _c_int, _c_void],
+    "ms_paged_attention_tiled_mfma_wide_chunk": [_c_int, _c_int, _c_int, _c_int],
     "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_activate": [_c_void, _c_void, _c_int, _c_ll, _c_int, _c_void],
     "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
@@ -544,6 +548,8 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, value_dim: in
     return page
 
 
+TILED_ROWS = 64  # query rows (tokens x the heads of a group) a block of the tiled attention kernels owns
+MFMA_DECODE_GROUP = 8  # query heads per key head from which single-token rows run the tiled matrix-core kernel too
 GENERIC_MAX_HEAD_DIM = 1024  # head sizes the generic attention kernel takes (MAX_WIDE_HEAD_DIM in csrc/attention.hip)
 
 
@@ -729,6 +735,28 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
         extra = (float(softcap), _ptr(sinks), int(value_share), int(values_in_keys), int(out_f32))
         tile_tokens = 0 if special else lib.ms_paged_attention_tiled_tokens(num_heads // num_kv_heads, head_dim, dv)
         lens = getattr(batch, "row_lens", None)
+        group = num_heads // num_kv_heads
+        wide = (special and lens is not None and qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and not values_in_keys
+                and lib.ms_paged_attention_tiled_mfma_wide_chunk(group, head_dim, dv, page))
+        # On the matrix cores: rows that bring several tokens, and single-token rows too where a key head serves so many
+        # query heads that they fill a wave's 16 rows.
+        wide_rows = t if (wide and group >= MFMA_DECODE_GROUP) else (t - n_dec if wide else 0)
+        if wide_rows:
+            all_rows = wide_rows == t
+            if not all_rows and n_dec:
+                _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES,
+                                                      *extra, _stream()), "paged_attention")
+            first, count, tiles = _tiles_of_rows(batch, TILED_ROWS // group, qkv.device, all_rows)
+            if block_table.shape[1] % 4:  # the kernel reads the four page ids of a key tile at once
+                padded = torch.zeros((block_table.shape[0], -(-block_table.shape[1] // 4) * 4), dtype=I32, device=block_table.device)
+                padded[:, : block_table.shape[1]] = block_table
+                common = (padded.data_ptr(), padded.shape[1])
+            _check(lib.ms_paged_attention_tiled_mfma_wide(
+                qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(), tiles,
+                batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), int(out_f32), num_heads, num_kv_heads, head_dim,
+                dv, page, float(scale), int(window), int(keep_first), float(softcap), _ptr(sinks), int(value_share), _stream()),
+                "paged_attention_tiled_mfma_wide")
+            return out
         if special and lens is not None and 0 < n_dec < t:
             # single-token rows walk their keys with several waves, the others with one wave per token and head
             _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES,
@@ -809,14 +837,32 @@ def _tiles_of(batch, tile_tokens: int, device):
     return build_prefill_tiles(batch.row_lens, batch.row_starts_host, tile_tokens, device)
 
 
-def build_prefill_tiles(row_lens, row_starts, tile_tokens: int, device):
-    """Tiles of at most ``tile_tokens`` consecutive new tokens of the rows that bring several tokens:
-    ``(first flat token index [n], token count [n], n)`` on the device, the tile deepest into its
+def _tiles_of_rows(batch, tile_tokens: int, device, all_rows: bool):
+    """Tiles of the rows that bring several tokens, or, ``all_rows``, of every row (a single token is a tile of one).
+    A step of single tokens only gets its tiles from the device alone (one per token, in order), so that a captured
+    graph can replay them."""
+    if not all_rows:
+        return _tiles_of(batch, tile_tokens, device)
+    if batch.num_decode_tokens == batch.num_tokens:
+        key = ("single-token tiles",)
+        if key not in batch.memo:
+            n = batch.num_tokens
+            batch.memo[key] = (torch.arange(n, dtype=I32, device=device), torch.ones(n, dtype=I32, device=device), n)
+        return batch.memo[key]
+    key = ("tiles of all rows", tile_tokens)
+    if key not in batch.memo:
+        batch.memo[key] = build_prefill_tiles(batch.row_lens, batch.row_starts_host, tile_tokens, device, least=1)
+    return batch.memo[key]
+
+
+def build_prefill_tiles(row_lens, row_starts, tile_tokens: int, device, least: int = 2):
+    """Tiles of at most ``tile_tokens`` consecutive new tokens of the rows that bring several tokens (at least
+    ``least``): ``(first flat token index [n], token count [n], n)`` on the device, the tile deepest into its
     sequence (the most keys to visit) first."""
     tiles = []
     t = 0
     for n, s in zip(row_lens, row_starts):
-        if n > 1:
+        if n >= least:
             for a in range(0, n, tile_tokens):
                 tiles.append((s + min(n, a + tile_tokens), t + a, min(tile_tokens, n - a)))
         t += n
@@ -1107,12 +1153,14 @@ def map_difference_norm(a: torch.Tensor, groups: int, per_group: int, value_dim:
     return out
 
 
-def latent_prepare(x, q_col: int, kv_col: int | None, rope, rot: int, pairing: str, latent_weight, eps, slots, k_cache,
+def latent_prepare(x, q_col: int, kv_col: int | None, rope, rot: int, pairing: str, latent_weight, eps, slots, k_cache, v_cache,
                    heads: int, plain_dim: int, rot_dim: int, latent_dim: int, out_dtype):
     """From the float32 projection ``x``: every head's plain query part into ``q_plain [T, H Dn]``, its turned part into
     the last ``R`` columns of that head in ``q_full [T, H (C + R)]`` (the first ``C`` are left for the caller), and, with
-    ``kv_col``, the token's cache row ``[C + R]`` at ``slots``: the latent after an RMS norm (``latent_weight``) and the
-    turned shared key part. The first ``rot`` of the ``R`` elements turn by ``rope``'s angles. Returns ``(q_plain, q_full)``."""
+    ``kv_col``, the token's cache row ``[C + R]`` at ``slots`` (``k_cache [pages, 1, page, C + R]``): the latent after an
+    RMS norm (``latent_weight``) and the turned shared key part; the normed latent goes to ``v_cache [pages, 1, C, page]``
+    as well, as the token's value. The first ``rot`` of the ``R`` elements turn by ``rope``'s angles. Returns
+    ``(q_plain, q_full)``."""
     _dev(x, "x", F32, 2)
     t = x.shape[0]
     if out_dtype not in (F32, BF16):
@@ -1124,10 +1172,10 @@ def latent_prepare(x, q_col: int, kv_col: int | None, rope, rot: int, pairing: s
     w_bf16 = 0
     if kv_col is not None:
         _dev(slots, "slots", I32, 1)
-        _dev(k_cache, "k_cache", out_dtype, 4)
+        page = _check_special_caches(k_cache, v_cache, out_dtype, 1, latent_dim + rot_dim, latent_dim, 1, False)
         _dev(latent_weight, "latent_weight", (F32, BF16), 1)
-        if slots.shape[0] != t or tuple(k_cache.shape[1:]) != (1, k_cache.shape[2], latent_dim + rot_dim) or latent_weight.shape[0] != latent_dim:
-            raise ValueError("one slot per token, a cache of one head of C + R elements and a weight of C elements are needed")
+        if slots.shape[0] != t or latent_weight.shape[0] != latent_dim:
+            raise ValueError("one slot per token and a weight of C elements are needed")
         w_bf16 = int(latent_weight.dtype == BF16)
     q_plain = torch.empty((t, heads * plain_dim), dtype=out_dtype, device=x.device)
     q_full = torch.empty((t, heads * (latent_dim + rot_dim)), dtype=out_dtype, device=x.device)
@@ -1135,7 +1183,8 @@ def latent_prepare(x, q_col: int, kv_col: int | None, rope, rot: int, pairing: s
         x.data_ptr(), x.shape[1], int(q_col), -1 if kv_col is None else int(kv_col), _ptr(rope) if rot else None, int(rot),
         _pairing(pairing), _ptr(latent_weight) if kv_col is not None else None, w_bf16, float(eps), q_plain.data_ptr(),
         q_full.data_ptr(), _ptr(slots) if kv_col is not None else None, _ptr(k_cache) if kv_col is not None else None,
-        int(out_dtype == BF16), t, heads, plain_dim, rot_dim, latent_dim, _stream()), "latent_prepare")
+        _ptr(v_cache) if kv_col is not None else None, page if kv_col is not None else 1, int(out_dtype == BF16), t, heads, plain_dim,
+        rot_dim, latent_dim, _stream()), "latent_prepare")
     return q_plain, q_full
 
 

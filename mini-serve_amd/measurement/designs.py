@@ -1,11 +1,18 @@
 """Prefill and decode throughput of one architecture beside another of equal size: random weights, layers of the
-sizes real models have, the same step function for both. ``bench.py --design kakunex`` prints what this returns.
+sizes real models have, the same step function for both. ``bench.py --design kakunex`` (or ``fimolix``) prints what
+this returns.
 
 A *shape* fixes what the two share: width, query and key/value heads of 128 elements, feed-forward width, window,
 layers, vocabulary. The Kakunex model of a shape repeats (parallel, parallel, parallel, mlstm): window attention that
 keeps the first 4 keys beside a decaying linear attention, and a matrix-memory layer in every fourth place, each
 recurrent mixer with as many heads of 128 x 128 as the attention has query heads. The Qwen3 model of the same
-shape attends within the same window in every layer."""
+shape attends within the same window in every layer.
+
+The Fimolix model of a shape repeats (latent attention, differential attention, differential attention, latent
+attention that reads the first one's cache). Its differential attention has half the shape's heads, each with two maps
+of 128 and values of 256, so that its four projections have the sizes of the Qwen3 layer's; convolutions of 4 taps. Its
+latent attention has the shape's query heads with 128 plain and 64 rotated elements, values of 128 and a latent of 512
+per token, inside the shape's window."""
 
 from __future__ import annotations
 
@@ -47,7 +54,25 @@ def qwen3_config(s: dict) -> dict:
             "layer_types": ["sliding_attention"] * s["layers"]}
 
 
-DESIGNS = {"kakunex": kakunex_config, "qwen3": qwen3_config}
+LATENT, ROTATED = 512, 64
+
+
+def fimolix_config(s: dict) -> dict:
+    mlp = {"kind": "dense", "ff": s["ff"]}
+    maps = {"heads": s["heads"] // 2, "kv_heads": max(1, s["kv_heads"] // 2), "dim": HEAD, "vdim": 2 * HEAD, "scale": HEAD ** -0.5,
+            "softcap": 50.0, "conv": 4, "diff": 0.5}
+    latent = {"heads": s["heads"], "dim": HEAD, "rot_dim": ROTATED, "vdim": HEAD, "kv_rank": LATENT, "scale": (HEAD + ROTATED) ** -0.5,
+              "rot": {"base": 1e4, "dims": ROTATED}, "mask": {"size": s["window"]}}
+    layers = []
+    for i in range(s["layers"]):
+        if i % 4 in (1, 2):
+            layers.append({"type": "attention", "mixer": dict(maps), "mlp": mlp})
+        else:
+            layers.append({"type": "latent_attention", "mixer": dict(latent, **({"kv_from": i - 3} if i % 4 == 3 else {})), "mlp": mlp})
+    return {"architecture": "Fimolix", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "layers": layers}
+
+
+DESIGNS = {"kakunex": kakunex_config, "fimolix": fimolix_config, "qwen3": qwen3_config}
 
 
 def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: int, steps: int, warmup: int, say=lambda m: None) -> dict:

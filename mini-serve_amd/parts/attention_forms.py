@@ -15,8 +15,9 @@ that the query heads of one key head lie side by side: (key/value head, map, hea
 all heads share. A head's key is ``[W_uk c, shared part]``, its value ``W_uv c``. The products with ``W_uk`` and
 ``W_uv`` are moved to the query's side and behind the weighted sum: ``q_plain . (W_uk c) = (W_uk^T q_plain) . c``
 and ``sum_j p_j W_uv c_j = W_uv sum_j p_j c_j``. The attention kernel then sees ``heads`` query heads of ``C + R``
-elements over one key head whose rows ``[c, rotated part]`` are also the values (their first ``C`` elements), and the
-cache holds nothing but those rows. Options: a sliding ``window``, a learned sink per head in the softmax's
+elements over one key head whose rows are ``[c, rotated part]`` and whose values are ``c`` again. The cache holds
+those rows and, as the values, ``c`` once more with the tokens of one element side by side (the order in which the
+matrix cores take the second product's operand). Options: a sliding ``window``, a learned sink per head in the softmax's
 denominator (``sinks``), a sigmoid gate per head read off the mixer's input (``gate``), and ``shares_cache``: the
 layer has no projection of its own for the latent and reads the cache rows another layer wrote (its run-order entry
 names that layer's cache slot), with query, up-projections, window and the rest of its own.
@@ -210,7 +211,7 @@ class LatentAttention(Mixer):
             self.sink = tensors[n["sink"]].to(torch.float32).contiguous()
 
     def kv_need(self) -> KVNeed:
-        return KVNeed((CachePlane("k", 1, self.key_dim),), self.window)
+        return KVNeed((CachePlane("k", 1, self.key_dim), CachePlane("v", 1, self.latent_dim, token_minor=True)), self.window)
 
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
@@ -222,11 +223,11 @@ class LatentAttention(Mixer):
             raise ValueError(f"{rot.dim} rotated elements in a part of {self.rot_dim}")
         q_plain, q_full = ops.latent_prepare(
             x32, self.q_col, self.kv_col, rot.table if rot is not None else None, rot.dim if rot is not None else 0,
-            rot.pairing if rot is not None else "halves", self.dkv_norm, self.eps, cache.slots, cache.k, self.heads,
+            rot.pairing if rot is not None else "halves", self.dkv_norm, self.eps, cache.slots, cache.k, cache.v, self.heads,
             self.plain_dim, self.rot_dim, self.latent_dim, self.rt.dtype)
         ops.head_linear(q_plain, self.uk_t, q_full, 0)
-        a = ops.paged_attention(q_full, cache.k, None, cache.block_table, batch, self.heads, 1, self.key_dim, self.scale,
-                                self.window, self.latent_dim, sinks=self.sink, values_in_keys=True)
+        a = ops.paged_attention(q_full, cache.k, cache.v, cache.block_table, batch, self.heads, 1, self.key_dim, self.scale,
+                                self.window, self.latent_dim, sinks=self.sink)
         o = torch.empty((x.shape[0], self.heads * self.value_dim), dtype=self.rt.dtype, device=x.device)
         ops.head_linear(a, self.uv, o, 0)
         if self.gate:

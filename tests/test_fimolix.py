@@ -65,7 +65,8 @@ def test_run_order_and_cache_groups():
             if e.writes_cache:
                 needs[e.cache] = CacheSlotNeed(e.cache, kv, st)
         layout = CacheLayout.from_needs([needs[s] for s in sorted(needs)])
-        latent_slots = {s for g in layout.groups if len(g.planes) == 1 for s in g.slots}
+        kinds = {i: layer["type"] for i, layer in enumerate(FIMOLIX[name][0]["layers"])}
+        latent_slots = {s for g in layout.groups for s in g.slots if kinds[s] == "latent_attention"}
         assert latent_slots == set(windows), name
         for i, layer in enumerate(FIMOLIX[name][0]["layers"]):
             st = mixers[i].state_need()

@@ -204,17 +204,20 @@ def test_latent_preparation(heads, dn, r, c, rot, pairing, dtype):
         assert np.allclose(turn(x[:, kv_col + c : kv_col + c + r]), F.rotate_adjacent(x[:, kv_col + c : kv_col + c + r], pos, rot, base))
     slots = rng.permutation(5 * PAGE)[:T]
     kc = torch.zeros((6, 1, PAGE, c + r), dtype=dtype, device=DEV)
+    vc = torch.zeros((6, 1, c, PAGE), dtype=dtype, device=DEV)
     qp, qf = o.latent_prepare(dev(x), q_col, kv_col, dev(table) if rot else None, rot, pairing, dev(cw, dtype), eps,
-                              dev(slots, torch.int32), kc, heads, dn, r, c, dtype)
+                              dev(slots, torch.int32), kc, vc, heads, dn, r, c, dtype)
     q = x[:, q_col : q_col + heads * (dn + r)].reshape(T, heads, dn + r)
     close(qp, q[:, :, :dn].reshape(T, -1), dtype, "plain query parts")
     close(qf.view(T, heads, c + r)[:, :, c:], turn(q[:, :, dn:]), dtype, "turned query parts")
     rows = kc.view(-1, c + r)[dev(slots, torch.int64)]
     close(rows[:, :c], F.rms_norm(x[:, kv_col : kv_col + c], rounded(cw, dtype), eps), dtype, "latent")
     close(rows[:, c:], turn(x[:, kv_col + c : kv_col + c + r]), dtype, "shared key part")
+    values = vc[:, 0].permute(0, 2, 1).reshape(-1, c)[dev(slots, torch.int64)]  # the latent once more, tokens side by side
+    assert torch.equal(values, rows[:, :c])
     # a layer that keeps nothing: queries only, the cache stays as it is
     before = kc.clone()
-    o.latent_prepare(dev(x), q_col, None, dev(table) if rot else None, rot, pairing, None, eps, None, None, heads, dn, r, c, dtype)
+    o.latent_prepare(dev(x), q_col, None, dev(table) if rot else None, rot, pairing, None, eps, None, None, None, heads, dn, r, c, dtype)
     assert torch.equal(kc, before)
 
 
@@ -250,7 +253,8 @@ CUTS = ([400], [150] + [1] * 250, [2, 3, 64, 5, 2, 31, 1, 1, 190, 1, 100])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hq,hk,share,d,e,cap", [(8, 4, 2, 16, 24, 4.0), (6, 2, 2, 10, 6, 30.0), (4, 4, 2, 64, 64, 0.0), (2, 2, 1, 48, 96, 2.0)])
+@pytest.mark.parametrize("hq,hk,share,d,e,cap", [(8, 4, 2, 16, 24, 4.0), (6, 2, 2, 10, 6, 30.0), (4, 4, 2, 64, 64, 0.0), (2, 2, 1, 48, 96, 2.0),
+                                                 (8, 4, 2, 128, 256, 4.0), (4, 2, 2, 32, 48, 3.0), (16, 2, 2, 96, 32, 0.0)])
 def test_capped_scores_and_shared_values(hq, hk, share, d, e, cap, dtype):
     """Several key heads weigh one value head; scores are bounded. One far key per query head is made to stand out
     (beyond the cap's linear range), so that a lost key, a wrong head pairing or a missing cap moves the result."""
@@ -277,11 +281,14 @@ def test_capped_scores_and_shared_values(hq, hk, share, d, e, cap, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("h,d,e,size", [(3, 32, 24, 37), (2, 11, 9, 16), (2, 288, 272, 100), (4, 40, 40, 0), (1, 160, 128, 96)])
-def test_sinks_and_values_inside_the_keys(h, d, e, size, dtype):
-    """One key head whose rows are also the values, a window, a sink per head. The key just inside the window of the
-    last query and the one just outside are made to stand out: a window one token off shows. Pages that the window has
-    passed are given away (their table entries are no pages)."""
+@pytest.mark.parametrize("inside", [True, False])
+@pytest.mark.parametrize("h,d,e,size", [(3, 32, 24, 37), (2, 11, 9, 16), (2, 288, 272, 100), (4, 40, 40, 0), (1, 160, 128, 96),
+                                        (16, 160, 128, 96), (8, 576, 512, 150), (12, 64, 48, 20)])
+def test_sinks_a_window_and_values_that_repeat_the_keys(h, d, e, size, inside, dtype):
+    """One key head whose rows' first elements are also the values (read from the key rows themselves, or from a value
+    cache that repeats them), a window, a sink per head. The key just inside the window of the last query and the one
+    just outside are made to stand out: a window one token off shows. Pages that the window has passed are given away
+    (their table entries are no pages)."""
     o = ops()
     rng = np.random.default_rng(h * d)
     T, scale = 400, 0.25
@@ -296,18 +303,21 @@ def test_sinks_and_values_inside_the_keys(h, d, e, size, dtype):
     assert np.abs(none - want).max() > 0.05 * np.abs(want).max()
     pages = [int(p) for p in rng.permutation(30)[: -(-T // PAGE)]]
     kc = torch.zeros((31, 1, PAGE, d), dtype=dtype, device=DEV)
+    vc = None if inside else torch.zeros((31, 1, e, PAGE), dtype=dtype, device=DEV)
     for p in range(T):
         kc[pages[p // PAGE], 0, p % PAGE] = dev(k[p, 0], dtype)
-    kw = dict(num_heads=h, num_kv_heads=1, head_dim=d, scale=scale, window=size, value_dim=e, sinks=dev(sinks), values_in_keys=True)
+        if not inside:
+            vc[pages[p // PAGE], 0, :, p % PAGE] = dev(k[p, 0, :e], dtype)
+    kw = dict(num_heads=h, num_kv_heads=1, head_dim=d, scale=scale, window=size, value_dim=e, sinks=dev(sinks), values_in_keys=inside)
     for cuts in CUTS:
-        got = run_attention(o, dev(q.reshape(T, -1), dtype), kc, None, pages, cuts, T, **kw)
+        got = run_attention(o, dev(q.reshape(T, -1), dtype), kc, vc, pages, cuts, T, **kw)
         close(got, want.reshape(T, -1), dtype, f"cuts {cuts[:3]}", tol=2e-5 if dtype == torch.float32 else 6e-3)
     if size:  # the last tokens again, with every page before the window gone
         first_live = (T - 20 - size + 1) // PAGE
         gone = [-1 if i < first_live else p for i, p in enumerate(pages)]
         table = dev([gone + [0] * (-len(gone) % 4)], torch.int32)
         b = step_batch([20], [T - 20])
-        got = o.paged_attention(dev(q.reshape(T, -1), dtype)[T - 20 :].contiguous(), kc, None, table, b, **kw)
+        got = o.paged_attention(dev(q.reshape(T, -1), dtype)[T - 20 :].contiguous(), kc, vc, table, b, **kw)
         close(got, want.reshape(T, -1)[T - 20 :], dtype, "pages before the window given away", tol=2e-5 if dtype == torch.float32 else 6e-3)
 
 
@@ -505,7 +515,8 @@ def test_a_borrowed_cache_is_kept_as_long_as_its_widest_reader_needs(folders):
 
     for name, window in (("fxA", 33), ("fxB", 21), ("fxD", 40)):
         runner = ModelRunner(load_model(folders[name], "float32", DEV), kv_pool_tokens=64, max_running=1)
-        latent = [g for g in runner.layout.groups if len(g.planes) == 1]
+        layers = FIMOLIX[name][0]["layers"]
+        latent = [g for g in runner.layout.groups if layers[g.slots[0]]["type"] == "latent_attention"]
         assert [g.window for g in latent] == [window], name
         assert len(latent[0].slots) == 1  # the reader has no pages of its own
 
