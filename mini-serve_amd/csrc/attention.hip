@@ -694,19 +694,23 @@ __device__ __forceinline__ float tanh_fast(float x) {
 // the cache: a block's 64 query rows are what all its tiles share) instead of living in registers; a block owns DVC of a
 // head's Dv value elements (blockIdx.z names the run), so a head of 512 values is four blocks that each form the scores
 // again. The keys' loads are issued per run of 64 elements, two runs under way.
-template <int DVC>
+template <int DVC, bool SPLIT>
 __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
     float* __restrict__ out32, int Hq, int Hkv, int D, int Dv, float scale, int window, int keep_first, float softcap,
-    const float* __restrict__ sinks, int value_share) {
+    const float* __restrict__ sinks, int value_share, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int PS = WAVE + 4;  // floats between a wave's rows of weights
   __shared__ __attribute__((aligned(16))) float Pw[4][16][PS];
+  __shared__ float Mo[SPLIT ? 4 : 1][SPLIT ? 16 : 1][SPLIT ? DVC : 1];  // SPLIT: the waves' outputs, maxima and sums meet here
+  __shared__ float Mml[SPLIT ? 4 : 1][16][2];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
   const int kvh = blockIdx.y, g = Hq / Hkv, e0 = blockIdx.z * DVC;
   const int Hv = Hkv / value_share, vh = kvh / value_share;
-  const int first = tile_first[blockIdx.x], count = tile_count[blockIdx.x], rows = count * g;
+  const int tile = SPLIT ? blockIdx.x / splits : blockIdx.x, split = SPLIT ? blockIdx.x % splits : 0;
+  const int first = tile_first[tile], count = tile_count[tile], rows = count * g;
+  const int rb = SPLIT ? 0 : wave * 16;  // SPLIT: every wave holds the tile's (at most 16) rows and takes every fourth key tile
   const int* table = block_table + (size_t)token_row[first] * table_width;
   const int p_first = pos[first], p_last = p_first + count - 1;
   const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
@@ -714,12 +718,12 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   const int chunks = D / 32;
 
   // this lane's query row as the A operand: row 16 wave + l16, elements 32 kk + 8 grp .. + 7
-  const int qr = wave * 16 + l16;
+  const int qr = rb + l16;
   const bf16* qp = qr < rows ? q + (size_t)(first + qr / g) * q_stride + (size_t)(kvh * g + qr % g) * D + grp * 8 : nullptr;
   int pr[4], lor[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int row = wave * 16 + grp * 4 + r;
+    const int row = rb + grp * 4 + r;
     pr[r] = row < rows ? p_first + row / g : -1;
     lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
   }
@@ -737,7 +741,10 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   const int kept_tiles = (kept + WAVE - 1) / WAVE;
   const int first_window_tile = lo_first / WAVE > kept_tiles ? lo_first / WAVE : kept_tiles;
   const int tiles = kept_tiles + (p_last / WAVE - first_window_tile + 1);
-  for (int ti = 0; ti < tiles; ++ti) {
+  const int per_split = SPLIT ? (tiles + splits - 1) / splits : tiles;
+  const int t_begin = SPLIT ? split * per_split + wave : 0;
+  const int t_end = SPLIT ? ((split + 1) * per_split < tiles ? (split + 1) * per_split : tiles) : tiles;
+  for (int ti = t_begin; ti < t_end; ti += SPLIT ? 4 : 1) {
     const int j0 = (ti < kept_tiles ? ti : first_window_tile + (ti - kept_tiles)) * WAVE;
     const int4 pg4 = *reinterpret_cast<const int4*>(table + j0 / MFMA_PAGE);
     const int pages[4] = {pg4.x, pg4.y, pg4.z, pg4.w};
@@ -829,9 +836,58 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     }
     __builtin_amdgcn_wave_barrier();  // the weights have been read before the next tile's are written
   }
+  if (SPLIT) {
+    // the four waves' partial results, brought to one maximum in wave order
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (l16 == 0) {
+        Mml[wave][grp * 4 + r][0] = m_run[r];
+        Mml[wave][grp * 4 + r][1] = l_run[r];
+      }
+#pragma unroll
+      for (int et = 0; et < DVC / 16; ++et) Mo[wave][grp * 4 + r][et * 16 + l16] = o[et][r];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = grp * 4 + r;
+      float m_all = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, Mml[w][row][0]);
+      float l = 0.f;
+#pragma unroll
+      for (int et = 0; et < DVC / 16; ++et) o[et][r] = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float mw = Mml[w][row][0];
+        const float c = mw == -INFINITY ? 0.f : expf(mw - m_all);  // a wave without a visible key
+        l += Mml[w][row][1] * c;
+#pragma unroll
+        for (int et = 0; et < DVC / 16; ++et) o[et][r] += Mo[w][row][et * 16 + l16] * c;
+      }
+      m_run[r] = m_all;
+      l_run[r] = l;
+    }
+    if (splits > 1) {
+      // one part of the keys: unnormalised outputs, maximum and sum, for the merge kernel
+      const size_t slot = (((size_t)tile * Hkv + kvh) * gridDim.z + blockIdx.z) * splits + split;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = grp * 4 + r;
+        if (l16 == 0) {
+          part_ml[(slot * 16 + row) * 2] = m_run[r];
+          part_ml[(slot * 16 + row) * 2 + 1] = l_run[r];
+        }
+#pragma unroll
+        for (int et = 0; et < DVC / 16; ++et) part_o[(slot * 16 + row) * DVC + et * 16 + l16] = o[et][r];
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int row = wave * 16 + grp * 4 + r;
+    const int row = rb + grp * 4 + r;
     if (row >= rows) continue;
     const int head = kvh * g + row % g;
     float inv = 1.f / l_run[r];
@@ -849,6 +905,41 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   }
 }
 
+// The parts of the SPLIT form into the result: per row the parts' maxima, sums and outputs are brought to one maximum
+// in ascending order of the parts, then the sink joins the denominator. One block per (tile, key head, run of values).
+template <int DVC>
+__global__ __launch_bounds__(256) void paged_attention_mfma_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ tile_first,
+    const int* __restrict__ tile_count, bf16* __restrict__ out, float* __restrict__ out32, int Hq, int Hkv, int Dv, int splits,
+    const float* __restrict__ sinks) {
+  const int tile = blockIdx.x, kvh = blockIdx.y, g = Hq / Hkv, e0 = blockIdx.z * DVC;
+  const int first = tile_first[tile], rows = tile_count[tile] * g;
+  const size_t slot0 = (((size_t)tile * Hkv + kvh) * gridDim.z + blockIdx.z) * splits;
+  for (int i = threadIdx.x; i < 16 * DVC; i += 256) {
+    const int row = i / DVC, e = i % DVC;
+    if (row >= rows) continue;
+    float m_all = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp) m_all = fmaxf(m_all, part_ml[((slot0 + sp) * 16 + row) * 2]);
+    float l = 0.f, acc = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float mw = part_ml[((slot0 + sp) * 16 + row) * 2];
+      const float c = mw == -INFINITY ? 0.f : expf(mw - m_all);
+      l += part_ml[((slot0 + sp) * 16 + row) * 2 + 1] * c;
+      acc += part_o[((slot0 + sp) * 16 + row) * DVC + e] * c;
+    }
+    const int head = kvh * g + row % g;
+    float inv = 1.f / l;
+    if (sinks) {
+      const float sink = sinks[head], m2 = fmaxf(m_all, sink);
+      const float c = expf(m_all - m2);
+      inv = c / (l * c + expf(sink - m2));
+    }
+    const size_t at = ((size_t)(first + row / g) * Hq + head) * Dv + e0 + e;
+    if (out32) out32[at] = acc * inv;
+    else out[at] = static_cast<bf16>(acc * inv);
+  }
+}
+
 // The run of value elements a block of the wide form owns (0: it does not take the shape): keys a multiple of 32,
 // values a multiple of 16, up to 64 query heads per key head, 16-token pages.
 extern "C" int ms_paged_attention_tiled_mfma_wide_chunk(int group, int D, int Dv, int page_size) {
@@ -862,21 +953,35 @@ extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, c
                                                   const int* block_table, int table_width, const int* tile_first,
                                                   const int* tile_count, int tiles, const int* token_row, const int* pos, void* out,
                                                   int out_f32, int Hq, int Hkv, int D, int Dv, int page_size, float scale, int window,
-                                                  int keep_first, float softcap, const float* sinks, int value_share, hipStream_t st) {
+                                                  int keep_first, float softcap, const float* sinks, int value_share, int splits,
+                                                  float* part_o, float* part_ml, hipStream_t st) {
   if (tiles <= 0) return MS_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || window < 0 || keep_first < 0 || table_width <= 0 || table_width % 4 || Hkv > 65535 ||
       q_stride < Hq * D || q_stride % 8 || tile_first == nullptr || tile_count == nullptr || !(softcap >= 0.f) || value_share < 1 ||
-      Hkv % value_share)
+      Hkv % value_share || splits < 0 || (splits > 1 && (part_o == nullptr || part_ml == nullptr)) || (splits > 0 && Hq / Hkv > 16))
     return MS_BAD_ARG;
   const int chunk = ms_paged_attention_tiled_mfma_wide_chunk(Hq / Hkv, D, Dv, page_size);
   if (chunk == 0 || Dv / chunk > 65535) return MS_UNSUPPORTED;
   if (window == 0) keep_first = 0;
-  dim3 grid(tiles, Hkv, Dv / chunk);
+  bf16* o16 = out_f32 ? nullptr : (bf16*)out;
+  float* o32 = out_f32 ? (float*)out : nullptr;
+  // splits == 0: tiles of up to 64 rows, a wave 16 of them. splits >= 1: every tile is one token (at most 16 rows); the
+  // block's waves share its key tiles, and `splits` blocks share a tile's keys, their parts meeting in the merge kernel.
+  dim3 grid(splits > 0 ? tiles * splits : tiles, Hkv, Dv / chunk);
 #define TW(CC)                                                                                                                 \
-  paged_attention_tiled_mfma_wide_kernel<CC><<<grid, 256, 0, st>>>(                                                            \
-      (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, pos, \
-      out_f32 ? nullptr : (bf16*)out, out_f32 ? (float*)out : nullptr, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks,   \
-      value_share)
+  do {                                                                                                                         \
+    if (splits > 0)                                                                                                            \
+      paged_attention_tiled_mfma_wide_kernel<CC, true><<<grid, 256, 0, st>>>(                                                  \
+          (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row,  \
+          pos, o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, splits, part_o, part_ml);      \
+    else                                                                                                                       \
+      paged_attention_tiled_mfma_wide_kernel<CC, false><<<grid, 256, 0, st>>>(                                                 \
+          (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row,  \
+          pos, o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, 1, nullptr, nullptr);          \
+    if (splits > 1)                                                                                                            \
+      paged_attention_mfma_merge_kernel<CC><<<dim3(tiles, Hkv, Dv / chunk), 256, 0, st>>>(part_o, part_ml, tile_first, tile_count,  \
+                                                                                         o16, o32, Hq, Hkv, Dv, splits, sinks); \
+  } while (0)
   if (chunk == 128) TW(128);
   else if (chunk == 64) TW(64);
   else if (chunk == 32) TW(32);

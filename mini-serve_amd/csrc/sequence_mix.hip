@@ -266,3 +266,75 @@ extern "C" int ms_activate(const float* x, void* out, int out_is_bf16, long long
   else activate_kernel<float><<<blocks, 256, 0, st>>>(x, (float*)out, (size_t)n, act);
   return launch_status();
 }
+
+// ---------------------------------------------------------------------------------------------
+// A matrix product per head in one launch, on the matrix cores: out[m][h * out_stride + col0 + n] = sum_k x[m][h * K + k] *
+// w[h][n][k], x [M, ld >= H K] and w [H, N, K] bfloat16, float32 sums (v_mfma_f32_16x16x32_bf16), the result bfloat16 or
+// float32. A block owns 64 rows x 64 columns of one head, a wave 16 of the rows; both operands come straight from
+// memory, 16 bytes a lane (the weights of a head are small and stay in the cache). K a multiple of 8.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hg_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hg_floatx4;
+
+__device__ __forceinline__ hg_bf16x8 hg_load(const bf16* p, bool ok) {
+  union { uint4 u; hg_bf16x8 v; } x;
+  x.u = ok ? *reinterpret_cast<const uint4*>(p) : make_uint4(0, 0, 0, 0);
+  return x.v;
+}
+
+__global__ __launch_bounds__(256) void head_gemm_bf16_kernel(const bf16* __restrict__ x, int ldx, const bf16* __restrict__ w,
+                                                             void* __restrict__ out, int ldc, int out_stride, int col0, int M, int N,
+                                                             int K, int out_f32) {
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
+  const int h = blockIdx.z, m0 = blockIdx.x * 64 + wave * 16, n0 = blockIdx.y * 64;
+  if (m0 >= M) return;
+  const bool row_ok = m0 + l16 < M;
+  const bf16* xp = x + (size_t)(m0 + l16) * ldx + (size_t)h * K + grp * 8;
+  const bf16* wp[4];
+  bool col_ok[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    col_ok[nt] = n0 + nt * 16 + l16 < N;
+    wp[nt] = w + ((size_t)h * N + n0 + nt * 16 + l16) * K + grp * 8;
+  }
+  hg_floatx4 acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) acc[nt] = hg_floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    hg_bf16x8 a[2], b[2][4];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int k = k0 + c * 32;
+      const bool in = k + grp * 8 < K;  // K is a multiple of 8: a lane's eight elements are all inside or all outside
+      a[c] = hg_load(xp + k, in && row_ok);
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) b[c][nt] = hg_load(wp[nt] + k, in && col_ok[nt]);
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c], b[c][nt], acc[nt], 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = m0 + grp * 4 + r;
+    if (m >= M) continue;
+    const size_t at = (size_t)m * ldc + (size_t)h * out_stride + col0 + n0 + l16;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      if (!col_ok[nt]) continue;
+      if (out_f32) ((float*)out)[at + nt * 16] = acc[nt][r];
+      else ((bf16*)out)[at + nt * 16] = static_cast<bf16>(acc[nt][r]);
+    }
+  }
+}
+
+extern "C" int ms_head_gemm_bf16(const void* x, int ldx, const void* w, void* out, int ldc, int out_stride, int col0, int out_f32,
+                                 int M, int H, int N, int K, hipStream_t st) {
+  if (M <= 0 || H <= 0 || N <= 0) return MS_OK;
+  if (K <= 0 || ldx < H * K || out_stride < col0 + N || ldc < H * out_stride || col0 < 0 || H > 65535 || (N + 63) / 64 > 65535)
+    return MS_BAD_ARG;
+  if (K % 8 || ldx % 8 || ((size_t)x % 16) || ((size_t)w % 16)) return MS_UNSUPPORTED;
+  head_gemm_bf16_kernel<<<dim3((M + 63) / 64, (N + 63) / 64, H), 256, 0, st>>>((const bf16*)x, ldx, (const bf16*)w, out, ldc, out_stride,
+                                                                             col0, M, N, K, out_f32);
+  return launch_status();
+}

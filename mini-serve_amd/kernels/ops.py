@@ -65,8 +65,9 @@ _SIGNATURES = {
                           _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_paged_attention_tiled_mfma_wide": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
                                            _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
-                                           _c_void, _c_int, _c_void],
+                                           _c_void, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_paged_attention_tiled_mfma_wide_chunk": [_c_int, _c_int, _c_int, _c_int],
+    "ms_head_gemm_bf16": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_activate": [_c_void, _c_void, _c_int, _c_ll, _c_int, _c_void],
     "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
@@ -549,6 +550,7 @@ def _check_caches(k_cache, v_cache, dtype, num_kv_heads, head_dim, value_dim: in
 
 
 TILED_ROWS = 64  # query rows (tokens x the heads of a group) a block of the tiled attention kernels owns
+MFMA_SPLIT_BLOCKS = 256  # blocks a step of single tokens aims for when it shares a token's keys among blocks
 MFMA_DECODE_GROUP = 8  # query heads per key head from which single-token rows run the tiled matrix-core kernel too
 GENERIC_MAX_HEAD_DIM = 1024  # head sizes the generic attention kernel takes (MAX_WIDE_HEAD_DIM in csrc/attention.hip)
 
@@ -747,6 +749,16 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
                 _check(lib.ms_paged_attention_generic(*generic, _ptr(batch.decode_tokens), *meta, n_dec, *shape, DECODE_GENERIC_WAVES,
                                                       *extra, _stream()), "paged_attention")
             first, count, tiles = _tiles_of_rows(batch, TILED_ROWS // group, qkv.device, all_rows)
+            splits, part_o, part_ml = 0, None, None
+            if all_rows and n_dec == t and group <= 16:
+                # a step of single tokens: a block's four waves share a token's key tiles, and so many blocks share them
+                # that the chip is full, each with at least a tile per wave
+                runs = dv // wide
+                key_tiles = -(-(min(batch.max_kv_len, window) if window else batch.max_kv_len) // 64) + 1
+                splits = max(1, min(key_tiles // 4, -(-MFMA_SPLIT_BLOCKS // (t * num_kv_heads * runs))))
+                if splits > 1:
+                    part_o = torch.empty((t * num_kv_heads * runs * splits * 16 * wide,), dtype=F32, device=qkv.device)
+                    part_ml = torch.empty((t * num_kv_heads * runs * splits * 16 * 2,), dtype=F32, device=qkv.device)
             if block_table.shape[1] % 4:  # the kernel reads the four page ids of a key tile at once
                 padded = torch.zeros((block_table.shape[0], -(-block_table.shape[1] // 4) * 4), dtype=I32, device=block_table.device)
                 padded[:, : block_table.shape[1]] = block_table
@@ -754,8 +766,8 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             _check(lib.ms_paged_attention_tiled_mfma_wide(
                 qkv.data_ptr(), qkv.shape[1], k_cache.data_ptr(), v_cache.data_ptr(), *common, first.data_ptr(), count.data_ptr(), tiles,
                 batch.token_row.data_ptr(), batch.positions.data_ptr(), out.data_ptr(), int(out_f32), num_heads, num_kv_heads, head_dim,
-                dv, page, float(scale), int(window), int(keep_first), float(softcap), _ptr(sinks), int(value_share), _stream()),
-                "paged_attention_tiled_mfma_wide")
+                dv, page, float(scale), int(window), int(keep_first), float(softcap), _ptr(sinks), int(value_share), splits,
+                _ptr(part_o), _ptr(part_ml), _stream()), "paged_attention_tiled_mfma_wide")
             return out
         if special and lens is not None and 0 < n_dec < t:
             # single-token rows walk their keys with several waves, the others with one wave per token and head
@@ -1215,8 +1227,9 @@ def activate(x: torch.Tensor, activation: str, out_dtype) -> torch.Tensor:
 def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_col: int = 0) -> torch.Tensor:
     """A matrix product per head: ``out[:, h * stride + out_col : ... + N] = x[:, h * K : (h + 1) * K] @ weights[h]^T`` with
     ``x [M, H K]``, ``weights [H, N, K]`` and ``out [M, H stride]`` (``stride = out.shape[1] / H >= out_col + N``; the other
-    columns of ``out`` stay). One launch of the engine's matrix kernels per head, over strided rows. Where a head's slice
-    does not start at a multiple of 16 bytes the head goes through contiguous copies."""
+    columns of ``out`` stay). bfloat16 weights with ``K`` a multiple of 8: one launch of a matrix-core kernel for all
+    heads. float32 weights: the true 32-bit product, one launch per head over strided rows. Other sizes: head by head
+    through contiguous copies."""
     _dev(x, "x", (F32, BF16), 2)
     _dev(weights, "weights", (F32, BF16), 3)
     _dev(out, "out", (F32, BF16), 2)
@@ -1228,24 +1241,21 @@ def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_c
         return out
     stride = out.shape[1] // h
     lib = library()
-    f32 = weights.dtype == F32
-    xa = cast(x, F32 if f32 else BF16)
-    xi, oi = xa.element_size(), out.element_size()
-    # the matrix-core kernels fetch 16 bytes at a time and store up to 16: every head's slices must start at such a multiple
-    direct = f32 or (k % 8 == 0 and (stride * oi) % 16 == 0 and (out_col * oi) % 16 == 0)
-    if not direct:
+    if weights.dtype == F32:
+        xa = cast(x, F32)
         for i in range(h):
-            y = linear(xa[:, i * k : (i + 1) * k].contiguous(), weights[i], out_dtype=out.dtype)
-            out[:, i * stride + out_col : i * stride + out_col + n].copy_(y)
+            _check(lib.ms_gemm_f32(xa.data_ptr() + i * k * 4, weights.data_ptr() + i * n * k * 4,
+                                   out.data_ptr() + (i * stride + out_col) * out.element_size(), 0 if out.dtype == F32 else 2, m, n, k,
+                                   h * k, out.shape[1], _stream()), "gemm_f32")
+        return out
+    xa = cast(x, BF16)
+    if k % 8 == 0:
+        _check(lib.ms_head_gemm_bf16(xa.data_ptr(), h * k, weights.data_ptr(), out.data_ptr(), out.shape[1], stride, int(out_col),
+                                     int(out.dtype == F32), m, h, n, k, _stream()), "head_gemm_bf16")
         return out
     for i in range(h):
-        xp = xa.data_ptr() + i * k * xi
-        wp = weights.data_ptr() + i * n * k * weights.element_size()
-        op = out.data_ptr() + (i * stride + out_col) * oi
-        if f32:
-            _check(lib.ms_gemm_f32(xp, wp, op, 0 if out.dtype == F32 else 2, m, n, k, h * k, out.shape[1], _stream()), "gemm_f32")
-        else:
-            _check(lib.ms_gemm_bf16(xp, wp, op, 1 if out.dtype == F32 else 0, m, n, k, h * k, out.shape[1], 1, _stream()), "gemm_bf16")
+        y = linear(xa[:, i * k : (i + 1) * k].contiguous(), weights[i], out_dtype=out.dtype)
+        out[:, i * stride + out_col : i * stride + out_col + n].copy_(y)
     return out
 
 
