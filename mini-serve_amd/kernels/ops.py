@@ -66,7 +66,7 @@ _SIGNATURES = {
     "ms_paged_attention_tiled_mfma_wide": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
                                            _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
                                            _c_void, _c_int, _c_int, _c_void, _c_void, _c_void],
-    "ms_paged_attention_tiled_mfma_wide_chunk": [_c_int, _c_int, _c_int, _c_int],
+    "ms_paged_attention_tiled_mfma_wide_chunk": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "ms_head_gemm_bf16": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_activate": [_c_void, _c_void, _c_int, _c_ll, _c_int, _c_void],
@@ -739,7 +739,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
         lens = getattr(batch, "row_lens", None)
         group = num_heads // num_kv_heads
         wide = (special and lens is not None and qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and not values_in_keys
-                and lib.ms_paged_attention_tiled_mfma_wide_chunk(group, head_dim, dv, page))
+                and lib.ms_paged_attention_tiled_mfma_wide_chunk(group, head_dim, dv, page, 1))
         # On the matrix cores: rows that bring several tokens, and single-token rows too where a key head serves so many
         # query heads that they fill a wave's 16 rows.
         wide_rows = t if (wide and group >= MFMA_DECODE_GROUP) else (t - n_dec if wide else 0)
@@ -753,7 +753,7 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
             if all_rows and n_dec == t and group <= 16:
                 # a step of single tokens: a block's four waves share a token's key tiles, and so many blocks share them
                 # that the chip is full, each with at least a tile per wave
-                runs = dv // wide
+                runs = dv // wide  # the run of values a block owns in a step of single tokens
                 key_tiles = -(-(min(batch.max_kv_len, window) if window else batch.max_kv_len) // 64) + 1
                 splits = max(1, min(key_tiles // 4, -(-MFMA_SPLIT_BLOCKS // (t * num_kv_heads * runs))))
                 if splits > 1:
