@@ -706,10 +706,13 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   __shared__ float Mo[SPLIT ? 4 : 1][SPLIT ? 16 : 1][SPLIT ? DVC : 1];  // SPLIT: the waves' outputs, maxima and sums meet here
   __shared__ float Mml[SPLIT ? 4 : 1][16][2];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
-  const int kvh = blockIdx.y, g = Hq / Hkv, e0 = blockIdx.z * DVC;
+  // SPLIT: a tile is one token, and a block owns up to 16 of a key head's query heads (blockIdx.y names key head and run)
+  const int g = Hq / Hkv, e0 = blockIdx.z * DVC, runs16 = SPLIT ? (g + 15) / 16 : 1;
+  const int kvh = blockIdx.y / runs16, hoff = (blockIdx.y % runs16) * 16;
   const int Hv = Hkv / value_share, vh = kvh / value_share;
   const int tile = SPLIT ? blockIdx.x / splits : blockIdx.x, split = SPLIT ? blockIdx.x % splits : 0;
-  const int first = tile_first[tile], count = tile_count[tile], rows = count * g;
+  const int first = tile_first[tile], count = SPLIT ? 1 : tile_count[tile];
+  const int rows = SPLIT ? (g - hoff < 16 ? g - hoff : 16) : count * g;
   const int rb = SPLIT ? 0 : wave * 16;  // SPLIT: every wave holds the tile's (at most 16) rows and takes every fourth key tile
   const int* table = block_table + (size_t)token_row[first] * table_width;
   const int p_first = pos[first], p_last = p_first + count - 1;
@@ -719,12 +722,15 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
 
   // this lane's query row as the A operand: row 16 wave + l16, elements 32 kk + 8 grp .. + 7
   const int qr = rb + l16;
-  const bf16* qp = qr < rows ? q + (size_t)(first + qr / g) * q_stride + (size_t)(kvh * g + qr % g) * D + grp * 8 : nullptr;
+  const bf16* qp = nullptr;
+  if (qr < rows)
+    qp = SPLIT ? q + (size_t)first * q_stride + (size_t)(kvh * g + hoff + qr) * D + grp * 8
+               : q + (size_t)(first + qr / g) * q_stride + (size_t)(kvh * g + qr % g) * D + grp * 8;
   int pr[4], lor[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int row = rb + grp * 4 + r;
-    pr[r] = row < rows ? p_first + row / g : -1;
+    pr[r] = row < rows ? (SPLIT ? p_first : p_first + row / g) : -1;
     lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
   }
   float m_run[4];
@@ -871,7 +877,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     }
     if (splits > 1) {
       // one part of the keys: unnormalised outputs, maximum and sum, for the merge kernel
-      const size_t slot = (((size_t)tile * Hkv + kvh) * gridDim.z + blockIdx.z) * splits + split;
+      const size_t slot = (((size_t)tile * gridDim.y + blockIdx.y) * gridDim.z + blockIdx.z) * splits + split;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = grp * 4 + r;
@@ -889,14 +895,14 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   for (int r = 0; r < 4; ++r) {
     const int row = rb + grp * 4 + r;
     if (row >= rows) continue;
-    const int head = kvh * g + row % g;
+    const int head = SPLIT ? kvh * g + hoff + row : kvh * g + row % g;
     float inv = 1.f / l_run[r];
     if (sinks) {  // exp(sink) joins the denominator: both are brought to the larger of the two maxima first
       const float sink = sinks[head], m_all = fmaxf(m_run[r], sink);
       const float c = expf(m_run[r] - m_all);
       inv = c / (l_run[r] * c + expf(sink - m_all));
     }
-    const size_t at = ((size_t)(first + row / g) * Hq + head) * Dv + e0;
+    const size_t at = ((size_t)(SPLIT ? first : first + row / g) * Hq + head) * Dv + e0;
 #pragma unroll
     for (int et = 0; et < DVC / 16; ++et) {
       if (out32) out32[at + et * 16 + l16] = o[et][r] * inv;
@@ -906,37 +912,46 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
 }
 
 // The parts of the SPLIT form into the result: per row the parts' maxima, sums and outputs are brought to one maximum
-// in ascending order of the parts, then the sink joins the denominator. One block per (tile, key head, run of values).
+// in ascending order of the parts, then the sink joins the denominator. One block per (token, key head and run of 16
+// query heads, run of values).
 template <int DVC>
 __global__ __launch_bounds__(256) void paged_attention_mfma_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ tile_first,
-    const int* __restrict__ tile_count, bf16* __restrict__ out, float* __restrict__ out32, int Hq, int Hkv, int Dv, int splits,
-    const float* __restrict__ sinks) {
-  const int tile = blockIdx.x, kvh = blockIdx.y, g = Hq / Hkv, e0 = blockIdx.z * DVC;
-  const int first = tile_first[tile], rows = tile_count[tile] * g;
-  const size_t slot0 = (((size_t)tile * Hkv + kvh) * gridDim.z + blockIdx.z) * splits;
-  for (int i = threadIdx.x; i < 16 * DVC; i += 256) {
-    const int row = i / DVC, e = i % DVC;
-    if (row >= rows) continue;
+    bf16* __restrict__ out, float* __restrict__ out32, int Hq, int Hkv, int Dv, int splits, const float* __restrict__ sinks) {
+  extern __shared__ float coef[];  // [16 rows][splits + 1]: each part's factor, then the factor of the whole
+  const int tile = blockIdx.x, g = Hq / Hkv, e0 = blockIdx.z * DVC, runs16 = (g + 15) / 16;
+  const int kvh = blockIdx.y / runs16, hoff = (blockIdx.y % runs16) * 16;
+  const int first = tile_first[tile], rows = g - hoff < 16 ? g - hoff : 16;
+  const size_t slot0 = (((size_t)tile * gridDim.y + blockIdx.y) * gridDim.z + blockIdx.z) * splits;
+  if (threadIdx.x < 16 && threadIdx.x < rows) {
+    const int row = threadIdx.x;
     float m_all = -INFINITY;
     for (int sp = 0; sp < splits; ++sp) m_all = fmaxf(m_all, part_ml[((slot0 + sp) * 16 + row) * 2]);
-    float l = 0.f, acc = 0.f;
+    float l = 0.f;
     for (int sp = 0; sp < splits; ++sp) {
       const float mw = part_ml[((slot0 + sp) * 16 + row) * 2];
-      const float c = mw == -INFINITY ? 0.f : expf(mw - m_all);
+      const float c = mw == -INFINITY ? 0.f : expf(mw - m_all);  // a part without a visible key
+      coef[row * (splits + 1) + sp] = c;
       l += part_ml[((slot0 + sp) * 16 + row) * 2 + 1] * c;
-      acc += part_o[((slot0 + sp) * 16 + row) * DVC + e] * c;
     }
-    const int head = kvh * g + row % g;
     float inv = 1.f / l;
     if (sinks) {
-      const float sink = sinks[head], m2 = fmaxf(m_all, sink);
+      const float sink = sinks[kvh * g + hoff + row], m2 = fmaxf(m_all, sink);
       const float c = expf(m_all - m2);
       inv = c / (l * c + expf(sink - m2));
     }
-    const size_t at = ((size_t)(first + row / g) * Hq + head) * Dv + e0 + e;
-    if (out32) out32[at] = acc * inv;
-    else out[at] = static_cast<bf16>(acc * inv);
+    coef[row * (splits + 1) + splits] = inv;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 16 * DVC; i += 256) {
+    const int row = i / DVC, e = i % DVC;
+    if (row >= rows) continue;
+    float acc = 0.f;
+    for (int sp = 0; sp < splits; ++sp) acc += part_o[((slot0 + sp) * 16 + row) * DVC + e] * coef[row * (splits + 1) + sp];
+    const size_t at = ((size_t)first * Hq + (kvh * g + hoff + row)) * Dv + e0 + e;
+    const float v = acc * coef[row * (splits + 1) + splits];
+    if (out32) out32[at] = v;
+    else out[at] = static_cast<bf16>(v);
   }
 }
 
@@ -961,16 +976,19 @@ extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, c
   if (tiles <= 0) return MS_OK;
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv || window < 0 || keep_first < 0 || table_width <= 0 || table_width % 4 || Hkv > 65535 ||
       q_stride < Hq * D || q_stride % 8 || tile_first == nullptr || tile_count == nullptr || !(softcap >= 0.f) || value_share < 1 ||
-      Hkv % value_share || splits < 0 || (splits > 1 && (part_o == nullptr || part_ml == nullptr)) || (splits > 0 && Hq / Hkv > 16))
+      Hkv % value_share || splits < 0 || (splits > 1 && (part_o == nullptr || part_ml == nullptr)))
     return MS_BAD_ARG;
   const int chunk = ms_paged_attention_tiled_mfma_wide_chunk(Hq / Hkv, D, Dv, page_size, splits > 0);
   if (chunk == 0 || Dv / chunk > 65535) return MS_UNSUPPORTED;
   if (window == 0) keep_first = 0;
   bf16* o16 = out_f32 ? nullptr : (bf16*)out;
   float* o32 = out_f32 ? (float*)out : nullptr;
-  // splits == 0: tiles of up to 64 rows, a wave 16 of them. splits >= 1: every tile is one token (at most 16 rows); the
-  // block's waves share its key tiles, and `splits` blocks share a tile's keys, their parts meeting in the merge kernel.
-  dim3 grid(splits > 0 ? tiles * splits : tiles, Hkv, Dv / chunk);
+  // splits == 0: tiles of up to 64 rows, a wave 16 of them. splits >= 1: every tile is one token; a block owns up to 16 of
+  // a key head's query heads, its waves share the key tiles, and `splits` blocks share a token's keys, their parts meeting
+  // in the merge kernel.
+  const int runs16 = (Hq / Hkv + 15) / 16;
+  if ((long)Hkv * runs16 > 65535) return MS_BAD_ARG;
+  dim3 grid(splits > 0 ? tiles * splits : tiles, splits > 0 ? Hkv * runs16 : Hkv, Dv / chunk);
 #define TW(CC)                                                                                                                 \
   do {                                                                                                                         \
     if (splits > 0)                                                                                                            \
@@ -982,8 +1000,8 @@ extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, c
           (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row,  \
           pos, o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, 1, nullptr, nullptr);          \
     if (splits > 1)                                                                                                            \
-      paged_attention_mfma_merge_kernel<CC><<<dim3(tiles, Hkv, Dv / chunk), 256, 0, st>>>(part_o, part_ml, tile_first, tile_count,  \
-                                                                                         o16, o32, Hq, Hkv, Dv, splits, sinks); \
+      paged_attention_mfma_merge_kernel<CC><<<dim3(tiles, Hkv * runs16, Dv / chunk), 256, 16 * (splits + 1) * sizeof(float), st>>>( \
+          part_o, part_ml, tile_first, o16, o32, Hq, Hkv, Dv, splits, sinks);                                                   \
   } while (0)
   if (chunk == 256) {
     paged_attention_tiled_mfma_wide_kernel<256, false><<<grid, 256, 0, st>>>(

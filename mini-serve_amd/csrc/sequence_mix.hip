@@ -14,7 +14,9 @@
 //   of position starts - (taps - 1) + i. Positions of this step come from x itself (the step's rows are consecutive).
 //   Norm: y / sqrt(mean(y^2) + eps) * w over each group, w [D] shared by all groups (nullptr: no norm).
 //   Keys [pages, Gk, page_size, D]; values transposed within the page, [pages, Hv, Dv, page_size].
-// One block per token; the convolved row lies in LDS.
+// A wave owns one unit of one token: a group of D query or key channels, or a head's Dv value channels (a lane holds
+// up to CONV_PER of them, 64 apart); a block four units.
+#define CONV_PER 16
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void conv_norm_store_kernel(
     const float* __restrict__ x, int ld, const TW* __restrict__ cw, int taps, const float* __restrict__ state,
@@ -22,41 +24,51 @@ __global__ __launch_bounds__(256) void conv_norm_store_kernel(
     const int* __restrict__ row_start, const int* __restrict__ starts, const TW* __restrict__ qw, const TW* __restrict__ kw,
     float eps, T* __restrict__ q_out, const int* __restrict__ slots, T* __restrict__ kc, T* __restrict__ vc, int Gq, int Gk,
     int Hv, int D, int Dv, int page_size) {
-  extern __shared__ float y[];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int u = blockIdx.y * (256 / WAVE) + wave;
+  if (u >= Gq + Gk + Hv) return;
   const int t = blockIdx.x, b = token_row[t], p = pos[t];
   const int start = starts[b], first = row_start[b];
-  const int nq = Gq * D, nk = Gk * D, nv = Hv * Dv, C = nq + nk + nv;
+  const int nq = Gq * D, nk = Gk * D, C = nq + nk + Hv * Dv;
+  const bool is_q = u < Gq, is_v = u >= Gq + Gk;
+  const int n = is_v ? Dv : D;
+  const int cb = is_v ? nq + nk + (u - Gq - Gk) * Dv : u * D;  // the key groups follow the query groups
   const float* old = state + (size_t)state_slots[b] * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  float y[CONV_PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < CONV_PER; ++i) {
+    const int d = lane + i * WAVE;
+    y[i] = 0.f;
+    if (d >= n) continue;
+    const int c = cb + d;
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int sp = p - taps + 1 + j;
       if (sp < 0) continue;
-      const float u = sp >= start ? x[(size_t)(first + sp - start) * ld + c] : old[(size_t)(taps - 1 - (start - sp)) * C + c];
-      acc = fmaf(to_f32(cw[(size_t)c * taps + j]), u, acc);
+      const float v = sp >= start ? x[(size_t)(first + sp - start) * ld + c] : old[(size_t)(taps - 1 - (start - sp)) * C + c];
+      acc = fmaf(to_f32(cw[(size_t)c * taps + j]), v, acc);
     }
-    y[c] = acc;
+    y[i] = acc;
+    ss += acc * acc;
   }
-  __syncthreads();
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int s = slots[t], page = s / page_size, off = s % page_size;
-  for (int g = wave; g < Gq + Gk; g += 256 / WAVE) {
-    const bool is_q = g < Gq;
-    const float* src = y + (size_t)g * D;  // the key groups follow the query groups
-    const TW* w = is_q ? qw : kw;
-    float r = 1.f;
-    if (w) {
-      float ss = 0.f;
-      for (int d = lane; d < D; d += WAVE) ss += src[d] * src[d];
-      r = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+  if (is_v) {
+    T* dst = vc + ((size_t)page * Hv + (u - Gq - Gk)) * Dv * page_size + off;
+#pragma unroll
+    for (int i = 0; i < CONV_PER; ++i) {
+      const int e = lane + i * WAVE;
+      if (e < n) dst[(size_t)e * page_size] = from_f32<T>(y[i]);
     }
-    T* dst = is_q ? q_out + (size_t)t * nq + (size_t)g * D
-                  : kc + (((size_t)page * Gk + (g - Gq)) * page_size + off) * D;
-    for (int d = lane; d < D; d += WAVE) dst[d] = from_f32<T>(w ? src[d] * r * to_f32(w[d]) : src[d]);
+    return;
   }
-  for (int i = threadIdx.x; i < nv; i += 256) {
-    const int h = i / Dv, e = i % Dv;
-    vc[(((size_t)page * Hv + h) * Dv + e) * page_size + off] = from_f32<T>(y[nq + nk + i]);
+  const TW* w = is_q ? qw : kw;
+  const float r = w ? 1.f / sqrtf(wave_sum(ss) / (float)D + eps) : 1.f;
+  T* dst = is_q ? q_out + (size_t)t * nq + (size_t)u * D : kc + (((size_t)page * Gk + (u - Gq)) * page_size + off) * D;
+#pragma unroll
+  for (int i = 0; i < CONV_PER; ++i) {
+    const int d = lane + i * WAVE;
+    if (d < n) dst[d] = from_f32<T>(w ? y[i] * r * to_f32(w[d]) : y[i]);
   }
 }
 
@@ -89,17 +101,14 @@ extern "C" int ms_conv_norm_store(const float* x, int ld, const void* cw, int w_
   if (taps < 1 || Gq <= 0 || Gk <= 0 || Hv <= 0 || D <= 0 || Dv <= 0 || page_size <= 0 || ld < C || rows <= 0 || rows > 65535 ||
       !(eps >= 0.f) || (taps > 1 && state == nullptr) || slots == nullptr || (qw == nullptr) != (kw == nullptr))
     return MS_BAD_ARG;
-  const size_t lds = (size_t)C * sizeof(float);
-  if (lds > 160 * 1024 - 4096) return MS_UNSUPPORTED;
+  if (D > CONV_PER * WAVE || Dv > CONV_PER * WAVE) return MS_UNSUPPORTED;
+  const int units = Gq + Gk + Hv;
+  if ((units + 3) / 4 > 65535) return MS_BAD_ARG;
+  const dim3 grid(tokens, (units + 3) / 4);
 #define CV(T, TW)                                                                                                             \
-  do {                                                                                                                        \
-    if (lds > 48 * 1024 && hipFuncSetAttribute((const void*)conv_norm_store_kernel<T, TW>,                                    \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)            \
-      return MS_LAUNCH_FAILED;                                                                                                \
-    conv_norm_store_kernel<T, TW><<<tokens, 256, lds, st>>>(x, ld, (const TW*)cw, taps, state, state_slots, token_row, pos,    \
-                                                            row_start, starts, (const TW*)qw, (const TW*)kw, eps, (T*)q_out,  \
-                                                            slots, (T*)kc, (T*)vc, Gq, Gk, Hv, D, Dv, page_size);             \
-  } while (0)
+  conv_norm_store_kernel<T, TW><<<grid, 256, 0, st>>>(x, ld, (const TW*)cw, taps, state, state_slots, token_row, pos, row_start, \
+                                                      starts, (const TW*)qw, (const TW*)kw, eps, (T*)q_out, slots, (T*)kc, (T*)vc, \
+                                                      Gq, Gk, Hv, D, Dv, page_size)
   if (out_is_bf16) {
     if (w_is_bf16) CV(bf16, bf16); else CV(bf16, float);
   } else {

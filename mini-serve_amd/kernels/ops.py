@@ -740,9 +740,11 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
         group = num_heads // num_kv_heads
         wide = (special and lens is not None and qkv.dtype == BF16 and qkv.shape[1] % 8 == 0 and not values_in_keys
                 and lib.ms_paged_attention_tiled_mfma_wide_chunk(group, head_dim, dv, page, 1))
-        # On the matrix cores: rows that bring several tokens, and single-token rows too where a key head serves so many
-        # query heads that they fill a wave's 16 rows.
-        wide_rows = t if (wide and group >= MFMA_DECODE_GROUP) else (t - n_dec if wide else 0)
+        # On the matrix cores: rows that bring several tokens; single-token rows too where a key head serves so many query
+        # heads that they fill a wave's 16 rows, or where the step has no other rows (its tokens' keys are then shared
+        # among waves and blocks, which pays whatever the group's size).
+        single_too = wide and (group >= MFMA_DECODE_GROUP or n_dec == t)
+        wide_rows = t if single_too else (t - n_dec if wide else 0)
         if wide_rows:
             all_rows = wide_rows == t
             if not all_rows and n_dec:
@@ -750,15 +752,16 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
                                                       *extra, _stream()), "paged_attention")
             first, count, tiles = _tiles_of_rows(batch, TILED_ROWS // group, qkv.device, all_rows)
             splits, part_o, part_ml = 0, None, None
-            if all_rows and n_dec == t and group <= 16:
+            if all_rows and n_dec == t:
                 # a step of single tokens: a block's four waves share a token's key tiles, and so many blocks share them
                 # that the chip is full, each with at least a tile per wave
+                heads16 = num_kv_heads * -(-group // 16)  # a block owns up to 16 of a key head's query heads
                 runs = dv // wide  # the run of values a block owns in a step of single tokens
                 key_tiles = -(-(min(batch.max_kv_len, window) if window else batch.max_kv_len) // 64) + 1
-                splits = max(1, min(key_tiles // 4, -(-MFMA_SPLIT_BLOCKS // (t * num_kv_heads * runs))))
+                splits = max(1, min(key_tiles // 4, -(-MFMA_SPLIT_BLOCKS // (t * heads16 * runs))))
                 if splits > 1:
-                    part_o = torch.empty((t * num_kv_heads * runs * splits * 16 * wide,), dtype=F32, device=qkv.device)
-                    part_ml = torch.empty((t * num_kv_heads * runs * splits * 16 * 2,), dtype=F32, device=qkv.device)
+                    part_o = torch.empty((t * heads16 * runs * splits * 16 * wide,), dtype=F32, device=qkv.device)
+                    part_ml = torch.empty((t * heads16 * runs * splits * 16 * 2,), dtype=F32, device=qkv.device)
             if block_table.shape[1] % 4:  # the kernel reads the four page ids of a key tile at once
                 padded = torch.zeros((block_table.shape[0], -(-block_table.shape[1] // 4) * 4), dtype=I32, device=block_table.device)
                 padded[:, : block_table.shape[1]] = block_table

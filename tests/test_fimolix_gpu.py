@@ -283,7 +283,7 @@ def test_capped_scores_and_shared_values(hq, hk, share, d, e, cap, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("inside", [True, False])
 @pytest.mark.parametrize("h,d,e,size", [(3, 32, 24, 37), (2, 11, 9, 16), (2, 288, 272, 100), (4, 40, 40, 0), (1, 160, 128, 96),
-                                        (16, 160, 128, 96), (8, 576, 512, 150), (12, 64, 48, 20)])
+                                        (16, 160, 128, 96), (8, 576, 512, 150), (12, 64, 48, 20), (40, 96, 64, 70)])
 def test_sinks_a_window_and_values_that_repeat_the_keys(h, d, e, size, inside, dtype):
     """One key head whose rows' first elements are also the values (read from the key rows themselves, or from a value
     cache that repeats them), a window, a sink per head. The key just inside the window of the last query and the one
