@@ -690,11 +690,11 @@ __device__ __forceinline__ float tanh_fast(float x) {
 
 // The same kernel for heads of any size that is a multiple of 32 (keys) and 16 (values), and for the options of the
 // generic form: a soft cap on the scores, a sink per query head, key heads that share a value head, float32 results.
-// What differs: the key size D is a run-time number, and the query fragments are fetched again for every key tile (from
-// the cache: a block's 64 query rows are what all its tiles share) instead of living in registers; a block owns DVC of a
-// head's Dv value elements (blockIdx.z names the run), so a head of 512 values is four blocks that each form the scores
-// again. The keys' loads are issued per run of 64 elements, two runs under way.
-template <int DVC, bool SPLIT>
+// What differs: the key size D is a run-time number (the query fragments live in registers where D <= 32 NQ, NQ = 4 or
+// 18, and are fetched again for every key tile where it is larger); a block owns DVC of a
+// head's Dv value elements (blockIdx.z names the run), so a head of 512 values is two blocks that each form the scores
+// again. A tile's keys go through LDS once for the block's four waves.
+template <int DVC, bool SPLIT, int NQ>
 __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
@@ -705,6 +705,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   __shared__ __attribute__((aligned(16))) float Pw[4][16][PS];
   __shared__ float Mo[SPLIT ? 4 : 1][SPLIT ? 16 : 1][SPLIT ? DVC : 1];  // SPLIT: the waves' outputs, maxima and sums meet here
   __shared__ float Mml[SPLIT ? 4 : 1][16][2];
+  extern __shared__ __attribute__((aligned(16))) bf16 Ks[];  // not SPLIT: the tile's keys, [64][D + 8]
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
   // SPLIT: a tile is one token, and a block owns up to 16 of a key head's query heads (blockIdx.y names key head and run)
   const int g = Hq / Hkv, e0 = blockIdx.z * DVC, runs16 = SPLIT ? (g + 15) / 16 : 1;
@@ -733,6 +734,12 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     pr[r] = row < rows ? (SPLIT ? p_first : p_first + row / g) : -1;
     lor[r] = (window > 0 && pr[r] - window + 1 > 0) ? pr[r] - window + 1 : 0;
   }
+  // NQ > 0: the lane's query fragments live in registers (D <= 32 NQ); else they are fetched again for every key tile
+  bf16x8 qreg[NQ > 0 ? NQ : 1];
+  if (NQ > 0) {
+#pragma unroll
+    for (int kk = 0; kk < NQ; ++kk) qreg[kk] = (qp && kk < chunks) ? load_bf16x8(qp + kk * 32) : zero_bf16x8();
+  }
   float m_run[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) m_run[r] = -INFINITY;
@@ -744,6 +751,9 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
   for (int u = 0; u < 8; ++u) ones[u] = static_cast<bf16>(1.f);
   const float cap_in = softcap > 0.f ? scale / softcap : 0.f;
 
+  // where this thread's 16-byte runs of a key tile lie (not SPLIT: the tile goes through LDS)
+  const int key_runs = D / 8;
+  const int stage_key = threadIdx.x / key_runs, stage_run = threadIdx.x % key_runs, stage_dq = 256 / key_runs, stage_dr = 256 % key_runs;
   const int kept_tiles = (kept + WAVE - 1) / WAVE;
   const int first_window_tile = lo_first / WAVE > kept_tiles ? lo_first / WAVE : kept_tiles;
   const int tiles = kept_tiles + (p_last / WAVE - first_window_tile + 1);
@@ -764,29 +774,105 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
 #pragma unroll
       for (int et = 0; et < DVC / 16; ++et) vf[ks][et] = seen ? load_bf16x8(vp + (size_t)(et * 16 + l16) * MFMA_PAGE) : zero_bf16x8();
     }
-    const bf16* kp[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
-      const bool seen = j <= p_last && (j >= lo_first || j < kept) && pages[t] >= 0;
-      kp[t] = seen ? kc + (((size_t)pages[t] * Hkv + kvh) * MFMA_PAGE + l16) * D + grp * 8 : nullptr;
-    }
     floatx4 s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int kk = 0; kk < chunks; kk += 2) {
-      bf16x8 qf[2], kf[2][4];
+    if (SPLIT) {
+      // every wave has key tiles of its own: the keys come straight from memory, two runs of 32 elements under way
+      const bf16* kp[4];
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const bool in = kk + c < chunks;
-        qf[c] = (in && qp) ? load_bf16x8(qp + (kk + c) * 32) : zero_bf16x8();
-#pragma unroll
-        for (int t = 0; t < 4; ++t) kf[c][t] = (in && kp[t]) ? load_bf16x8(kp[t] + (kk + c) * 32) : zero_bf16x8();
+      for (int t = 0; t < 4; ++t) {
+        const int j = j0 + t * 16 + l16;  // this lane's key as the B operand
+        const bool seen = j <= p_last && (j >= lo_first || j < kept) && pages[t] >= 0;
+        kp[t] = seen ? kc + (((size_t)pages[t] * Hkv + kvh) * MFMA_PAGE + l16) * D + grp * 8 : nullptr;
       }
+      if (NQ > 0) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+        for (int kk = 0; kk < NQ; kk += 2) {
+          if (kk >= chunks) continue;  // the same for every lane; no break, so that the loop unrolls and qreg stays in registers
+          bf16x8 kf[2][4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], kf[c][t], s[t], 0, 0, 0);
+          for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              kf[c][t] = (kk + c < chunks && kp[t]) ? load_bf16x8(kp[t] + (kk + c) * 32) : zero_bf16x8();
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (kk + c < NQ) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qreg[kk + c < NQ ? kk + c : 0], kf[c][t], s[t], 0, 0, 0);
+        }
+      } else {
+        for (int kk = 0; kk < chunks; kk += 2) {
+          bf16x8 qf[2], kf[2][4];
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            const bool in = kk + c < chunks;
+            qf[c] = (in && qp) ? load_bf16x8(qp + (kk + c) * 32) : zero_bf16x8();
+#pragma unroll
+            for (int t = 0; t < 4; ++t) kf[c][t] = (in && kp[t]) ? load_bf16x8(kp[t] + (kk + c) * 32) : zero_bf16x8();
+          }
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], kf[c][t], s[t], 0, 0, 0);
+        }
+      }
+    } else {
+      // The block's waves share the tile's keys: all of them are fetched at once into LDS, 16 bytes a thread and load
+      // (rows D + 8 elements apart: the 16 lanes that read 16 keys' runs of 8 elements meet in no bank), so that a tile
+      // waits for memory once and not once per run of elements. The query fragments come from the cache, the next
+      // run's under way while this one is multiplied.
+      __syncthreads();  // the tile before has been read
+      const int ld = D + 8;
+      int jj = stage_key, c = stage_run;  // thread's first 16-byte run; the next is 256 runs on (no division in the loop)
+      for (int i0 = threadIdx.x; i0 < WAVE * key_runs; i0 += 6 * 256) {
+        uint4 got[6];
+        int at[6];
+#pragma unroll
+        for (int u = 0; u < 6; ++u) {
+          const int j = j0 + jj;
+          const int page = jj < 16 ? pg4.x : jj < 32 ? pg4.y : jj < 48 ? pg4.z : pg4.w;
+          at[u] = i0 + u * 256 < WAVE * key_runs ? jj * ld + c * 8 : -1;
+          got[u] = make_uint4(0, 0, 0, 0);
+          if (at[u] >= 0 && j <= p_last && (j >= lo_first || j < kept) && page >= 0)
+            got[u] = *reinterpret_cast<const uint4*>(kc + (((size_t)page * Hkv + kvh) * MFMA_PAGE + jj % MFMA_PAGE) * D + c * 8);
+          jj += stage_dq;
+          c += stage_dr;
+          if (c >= key_runs) {
+            c -= key_runs;
+            ++jj;
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 6; ++u)
+          if (at[u] >= 0) *reinterpret_cast<uint4*>(Ks + at[u]) = got[u];
+      }
+      bf16x8 qn = (NQ == 0 && qp && chunks > 0) ? load_bf16x8(qp) : zero_bf16x8();
+      __syncthreads();
+      if (NQ > 0) {
+#pragma unroll
+        for (int kk = 0; kk < NQ; ++kk) {
+          if (kk >= chunks) continue;  // no break: the loop unrolls and qreg stays in registers
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            union { uint4 u; bf16x8 v; } kf;
+            kf.u = *reinterpret_cast<const uint4*>(Ks + (size_t)(t * 16 + l16) * ld + kk * 32 + grp * 8);
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qreg[kk], kf.v, s[t], 0, 0, 0);
+          }
+        }
+      } else {
+        for (int kk = 0; kk < chunks; ++kk) {
+          const bf16x8 qf = qn;
+          qn = (qp && kk + 1 < chunks) ? load_bf16x8(qp + (kk + 1) * 32) : zero_bf16x8();
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            union { uint4 u; bf16x8 v; } kf;
+            kf.u = *reinterpret_cast<const uint4*>(Ks + (size_t)(t * 16 + l16) * ld + kk * 32 + grp * 8);
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf, kf.v, s[t], 0, 0, 0);
+          }
+        }
+      }
     }
     float corr[4];
 #pragma unroll
@@ -988,29 +1074,43 @@ extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, c
   // in the merge kernel.
   const int runs16 = (Hq / Hkv + 15) / 16;
   if ((long)Hkv * runs16 > 65535) return MS_BAD_ARG;
+  // the tile's keys in LDS (not with splits): 64 rows of D + 8 elements, beside 17 KB of weights
+  const size_t key_lds = (size_t)WAVE * (D + 8) * sizeof(bf16);
+  if (splits == 0 && key_lds > 140 * 1024) return MS_UNSUPPORTED;
   dim3 grid(splits > 0 ? tiles * splits : tiles, splits > 0 ? Hkv * runs16 : Hkv, Dv / chunk);
+  const int nq = D <= 128 ? 4 : D <= 576 ? 18 : 0;  // 32-element runs of a query the kernel keeps in registers
+#define TWQ(CC, SP, QQ)                                                                                                        \
+  paged_attention_tiled_mfma_wide_kernel<CC, SP, QQ><<<grid, 256, SP ? 0 : key_lds, st>>>(                                     \
+      (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, pos, \
+      o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, SP ? splits : 1, SP ? part_o : nullptr,     \
+      SP ? part_ml : nullptr)
 #define TW(CC)                                                                                                                 \
   do {                                                                                                                         \
-    if (splits > 0)                                                                                                            \
-      paged_attention_tiled_mfma_wide_kernel<CC, true><<<grid, 256, 0, st>>>(                                                  \
-          (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row,  \
-          pos, o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, splits, part_o, part_ml);      \
-    else                                                                                                                       \
-      paged_attention_tiled_mfma_wide_kernel<CC, false><<<grid, 256, 0, st>>>(                                                 \
-          (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row,  \
-          pos, o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, 1, nullptr, nullptr);          \
+    if (splits > 0) {                                                                                                          \
+      if (nq == 4) TWQ(CC, true, 4); else if (nq == 18) TWQ(CC, true, 18); else TWQ(CC, true, 0);                              \
+    } else {                                                                                                                   \
+      const void* fn = nq == 4 ? (const void*)paged_attention_tiled_mfma_wide_kernel<CC, false, 4>                             \
+                       : nq == 18 ? (const void*)paged_attention_tiled_mfma_wide_kernel<CC, false, 18>                         \
+                                  : (const void*)paged_attention_tiled_mfma_wide_kernel<CC, false, 0>;                         \
+      if (key_lds > 40 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)key_lds) != hipSuccess) \
+        return MS_LAUNCH_FAILED;                                                                                               \
+      if (nq == 4) TWQ(CC, false, 4); else if (nq == 18) TWQ(CC, false, 18); else TWQ(CC, false, 0);                           \
+    }                                                                                                                          \
     if (splits > 1)                                                                                                            \
       paged_attention_mfma_merge_kernel<CC><<<dim3(tiles, Hkv * runs16, Dv / chunk), 256, 16 * (splits + 1) * sizeof(float), st>>>( \
           part_o, part_ml, tile_first, o16, o32, Hq, Hkv, Dv, splits, sinks);                                                   \
   } while (0)
   if (chunk == 256) {
-    paged_attention_tiled_mfma_wide_kernel<256, false><<<grid, 256, 0, st>>>(
-        (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, pos,
-        o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, 1, nullptr, nullptr);
+    const void* fn = nq == 18 ? (const void*)paged_attention_tiled_mfma_wide_kernel<256, false, 18>
+                              : (const void*)paged_attention_tiled_mfma_wide_kernel<256, false, 0>;
+    if (key_lds > 40 * 1024 && hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)key_lds) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    if (nq == 4 || nq == 18) TWQ(256, false, 18); else TWQ(256, false, 0);
   } else if (chunk == 128) TW(128);
   else if (chunk == 64) TW(64);
   else if (chunk == 32) TW(32);
   else TW(16);
+#undef TWQ
 #undef TW
   return launch_status();
 }

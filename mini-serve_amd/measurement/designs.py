@@ -60,7 +60,7 @@ LATENT, ROTATED = 512, 64
 def fimolix_config(s: dict) -> dict:
     mlp = {"kind": "dense", "ff": s["ff"]}
     maps = {"heads": s["heads"] // 2, "kv_heads": max(1, s["kv_heads"] // 2), "dim": HEAD, "vdim": 2 * HEAD, "scale": HEAD ** -0.5,
-            "softcap": 50.0, "conv": 4, "diff": 0.5}
+            "softcap": 30.0, "conv": 4, "diff": 0.4}
     latent = {"heads": s["heads"], "dim": HEAD, "rot_dim": ROTATED, "vdim": HEAD, "kv_rank": LATENT, "scale": (HEAD + ROTATED) ** -0.5,
               "rot": {"base": 1e4, "dims": ROTATED}, "mask": {"size": s["window"]}}
     layers = []

@@ -253,7 +253,7 @@ CUTS = ([400], [150] + [1] * 250, [2, 3, 64, 5, 2, 31, 1, 1, 190, 1, 100])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("hq,hk,share,d,e,cap", [(8, 4, 2, 16, 24, 4.0), (6, 2, 2, 10, 6, 30.0), (4, 4, 2, 64, 64, 0.0), (2, 2, 1, 48, 96, 2.0),
+@pytest.mark.parametrize("hq,hk,share,d,e,cap", [(8, 4, 2, 16, 24, 4.0), (6, 2, 2, 10, 6, 30.0), (4, 4, 2, 64, 64, 0.0), (2, 2, 1, 40, 72, 2.0),
                                                  (8, 4, 2, 128, 256, 4.0), (4, 2, 2, 32, 48, 3.0), (16, 2, 2, 96, 32, 0.0)])
 def test_capped_scores_and_shared_values(hq, hk, share, d, e, cap, dtype):
     """Several key heads weigh one value head; scores are bounded. One far key per query head is made to stand out
@@ -282,8 +282,8 @@ def test_capped_scores_and_shared_values(hq, hk, share, d, e, cap, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("inside", [True, False])
-@pytest.mark.parametrize("h,d,e,size", [(3, 32, 24, 37), (2, 11, 9, 16), (2, 288, 272, 100), (4, 40, 40, 0), (1, 160, 128, 96),
-                                        (16, 160, 128, 96), (8, 576, 512, 150), (12, 64, 48, 20), (40, 96, 64, 70)])
+@pytest.mark.parametrize("h,d,e,size", [(3, 32, 24, 37), (2, 11, 9, 16), (2, 288, 272, 100), (4, 40, 40, 0), (1, 192, 160, 80),
+                                        (16, 192, 160, 80), (8, 576, 512, 150), (12, 64, 48, 20), (40, 96, 64, 70)])
 def test_sinks_a_window_and_values_that_repeat_the_keys(h, d, e, size, inside, dtype):
     """One key head whose rows' first elements are also the values (read from the key rows themselves, or from a value
     cache that repeats them), a window, a sink per head. The key just inside the window of the last query and the one
