@@ -169,6 +169,36 @@ extern "C" int ms_normed_mean_add(float* residual, const float* const* streams, 
   return launch_status();
 }
 
+// residual += rmsnorm(stream + pending) * w for one stream whose last matrix product left partial sums (`splits` slices
+// `stride` floats apart, added in ascending order): the sums are formed twice, once for the mean of squares and once for
+// the result, instead of being written out by a kernel of their own. stream may be nullptr (zero).
+template <typename TW>
+__global__ __launch_bounds__(256) void normed_add_pending_kernel(float* __restrict__ residual, const float* __restrict__ stream,
+                                                                 const float* __restrict__ parts, int splits, size_t stride,
+                                                                 const TW* __restrict__ w, int width, float eps) {
+  __shared__ float red[256 / WAVE];
+  const size_t row = (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int e = threadIdx.x; e < width; e += 256) {
+    const float v = (stream ? stream[row + e] : 0.f) + sum_splits(parts + row + e, splits, stride);
+    ss += v * v;
+  }
+  const float rstd = 1.f / sqrtf(block_sum<256>(ss, red) / (float)width + eps);
+  for (int e = threadIdx.x; e < width; e += 256) {
+    const float v = (stream ? stream[row + e] : 0.f) + sum_splits(parts + row + e, splits, stride);
+    residual[row + e] += v * rstd * to_f32(w[e]);
+  }
+}
+
+extern "C" int ms_normed_add_pending(float* residual, const float* stream, const float* parts, int splits, long long stride,
+                                     const void* w, int w_is_bf16, int tokens, int width, float eps, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (width <= 0 || splits < 1 || stride < (long long)tokens * width || parts == nullptr || !(eps >= 0.f)) return MS_BAD_ARG;
+  if (w_is_bf16) normed_add_pending_kernel<bf16><<<tokens, 256, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const bf16*)w, width, eps);
+  else normed_add_pending_kernel<float><<<tokens, 256, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const float*)w, width, eps);
+  return launch_status();
+}
+
 // ---------------------------------------------------------------------------------------------
 __global__ void scale_kernel(float* __restrict__ x, size_t n, float s) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

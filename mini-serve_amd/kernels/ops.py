@@ -29,6 +29,7 @@ _SIGNATURES = {
     "ms_layernorm": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
     "ms_group_rmsnorm_gate": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
     "ms_normed_mean_add": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void],
+    "ms_normed_add_pending": [_c_void, _c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_float, _c_void],
     "ms_scale": [_c_void, _c_ll, _c_float, _c_void],
     "ms_qkv_norm_rope_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int, _c_int,
                                _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -1041,6 +1042,27 @@ def normed_mean_add(residual: torch.Tensor, streams, weights, eps: float, coef: 
     wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
     _check(library().ms_normed_mean_add(residual.data_ptr(), sp, wp, int(weights[0].dtype == BF16), n, residual.shape[0],
                                         residual.shape[1], float(eps), float(coef), _stream()), "normed_mean_add")
+
+
+def normed_add(residual: torch.Tensor, stream: torch.Tensor | None, weight: torch.Tensor, eps: float, pending: SplitSum | None = None) -> None:
+    """``residual += rmsnorm(stream + pending) * weight`` row by row: one float32 stream of the residual's shape (None:
+    zero) and the partial sums its last matrix product may have left (summed inside the kernel, no kernel of their own)."""
+    if pending is None:
+        if stream is None:
+            raise ValueError("neither a stream nor a pending sum")
+        return normed_mean_add(residual, [stream], [weight], eps, 1.0)
+    _dev(residual, "residual", F32, 2)
+    _dev(weight, "weight", (F32, BF16), 1)
+    _check_split(pending, "pending", residual.shape)
+    if stream is not None:
+        _dev(stream, "stream", F32, 2)
+        if stream.shape != residual.shape:
+            raise ValueError("the stream must have the residual's shape")
+    if weight.shape[0] != residual.shape[1]:
+        raise ValueError("the weight must have the residual's width")
+    _check(library().ms_normed_add_pending(residual.data_ptr(), _ptr(stream), pending.parts.data_ptr(), pending.splits, pending.stride,
+                                           weight.data_ptr(), int(weight.dtype == BF16), residual.shape[0], residual.shape[1], float(eps),
+                                           _stream()), "normed_add_pending")
 
 
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:

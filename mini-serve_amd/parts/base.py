@@ -188,9 +188,10 @@ class Norm(Part):
         also brought up to date in place; with ``rows`` the stream is not read again and stays as it is."""
         raise NotImplementedError
 
-    def add_normed(self, residual, stream) -> None:
-        """``residual += norm(stream)`` row by row, both float32 and of one shape: the norm of a layer that norms
-        what a sublayer puts out instead of what it reads."""
+    def add_normed(self, residual, stream, pending=None) -> None:
+        """``residual += norm(stream + pending)`` row by row, both float32 and of one shape (``pending``: a sum the
+        sublayer left to be added to its stream): the norm of a layer that norms what a sublayer puts out instead of
+        what it reads."""
         raise NotImplementedError(f"norm {self.kind!r} cannot norm a sublayer's output into the residual stream")
 
 

@@ -102,8 +102,8 @@ class OutputNormBlock(Block):
     def _sublayer(self, run, norm, residual) -> None:
         ops = self.rt.ops
         own = torch.zeros_like(residual)
-        ops.add_pending(own, run(ops.cast(residual, self.rt.dtype), own))
-        norm.add_normed(residual, own)
+        pending = run(ops.cast(residual, self.rt.dtype), own)
+        norm.add_normed(residual, own, pending)  # the sublayer's output is its stream plus what it left pending
 
     def forward(self, residual, batch, cache, state, pending=None):
         self.rt.ops.add_pending(residual, pending)

@@ -40,8 +40,8 @@ class RMSNorm(Norm):
         Returns the compute dtype, ``[T or len(rows), width]``."""
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows, add)
 
-    def add_normed(self, residual, stream) -> None:
-        self.rt.ops.normed_mean_add(residual, [stream], [self.weight], self.eps, 1.0)
+    def add_normed(self, residual, stream, pending=None) -> None:
+        self.rt.ops.normed_add(residual, stream, self.weight, self.eps, pending)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

@@ -105,6 +105,16 @@ def test_config_refusals():
     assert config_from_dict(preset("fimolix-tiny")).to_spec().architecture == "Fimolix"
 
 
+def test_the_measured_shapes_are_valid_configurations():
+    from miniserve_amd.measurement.designs import SHAPES, fimolix_config
+
+    for name, shape in SHAPES.items():
+        spec = config_from_dict(fimolix_config(shape)).to_spec()
+        assert len(spec.layers) == shape["layers"], name
+        borrowed = [e for e in spec.run_order if not e.writes_cache]
+        assert len(borrowed) == shape["layers"] // 4 and all(e.cache == e.layer - 3 for e in borrowed)
+
+
 def test_a_spare_second_norm_loads_and_is_ignored(tmp_path):
     """A layer without a feed-forward has no use for a second norm; a checkpoint that carries one all the same loads."""
     from safetensors.torch import load_file, save_file

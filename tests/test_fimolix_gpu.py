@@ -78,6 +78,19 @@ def test_activation_without_a_gate(n, dtype):
         ops().activate(dev(x), "swiglu_clamped", dtype)
 
 
+@pytest.mark.parametrize("width", [5, 176, 600])
+def test_norm_of_a_sublayers_output_into_the_stream(width):
+    """``residual += y / rms(y) * w`` with ``y`` a stream, a stream plus partial sums of its last product, or partial sums
+    alone."""
+    rng = np.random.default_rng(width)
+    r, y, w = rng.normal(size=(6, width)), rng.normal(size=(6, width)) * 10, rng.normal(size=width) + 1
+    parts = rng.normal(size=(3, 6, width))
+    for stream, pending, total in ((y, None, y), (y, parts, y + parts.sum(0)), (None, parts, parts.sum(0))):
+        res = dev(r)
+        ops().normed_add(res, None if stream is None else dev(stream), dev(w), 1e-6, None if pending is None else ops().SplitSum(dev(pending)))
+        close(res, r + F.rms_norm(total, w, 1e-6), torch.float32)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,size", [(1, 1), (3, 7), (6, 80)])
 def test_gate_per_head(heads, size, dtype):
