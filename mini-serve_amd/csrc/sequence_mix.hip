@@ -281,6 +281,7 @@ extern "C" int ms_activate(const float* x, void* out, int out_is_bf16, long long
 // w[h][n][k], x [M, ld >= H K] and w [H, N, K] bfloat16, float32 sums (v_mfma_f32_16x16x32_bf16), the result bfloat16 or
 // float32. A block owns 64 rows x 64 columns of one head, a wave 16 of the rows; both operands come straight from
 // memory, 16 bytes a lane (the weights of a head are small and stay in the cache). K a multiple of 8.
+// gate (optional): float32 rows of stride gate_ld; head h's results of row m are multiplied by sigmoid(gate[m][gate_col + h]).
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hg_bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hg_floatx4;
 
@@ -292,7 +293,8 @@ __device__ __forceinline__ hg_bf16x8 hg_load(const bf16* p, bool ok) {
 
 __global__ __launch_bounds__(256) void head_gemm_bf16_kernel(const bf16* __restrict__ x, int ldx, const bf16* __restrict__ w,
                                                              void* __restrict__ out, int ldc, int out_stride, int col0, int M, int N,
-                                                             int K, int out_f32) {
+                                                             int K, int out_f32, const float* __restrict__ gate, int gate_ld,
+                                                             int gate_col) {
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
   const int h = blockIdx.z, m0 = blockIdx.x * 64 + wave * 16, n0 = blockIdx.y * 64;
   if (m0 >= M) return;
@@ -328,22 +330,24 @@ __global__ __launch_bounds__(256) void head_gemm_bf16_kernel(const bf16* __restr
     const int m = m0 + grp * 4 + r;
     if (m >= M) continue;
     const size_t at = (size_t)m * ldc + (size_t)h * out_stride + col0 + n0 + l16;
+    const float gm = gate ? 1.f / (1.f + expf(-gate[(size_t)m * gate_ld + gate_col + h])) : 1.f;
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       if (!col_ok[nt]) continue;
-      if (out_f32) ((float*)out)[at + nt * 16] = acc[nt][r];
-      else ((bf16*)out)[at + nt * 16] = static_cast<bf16>(acc[nt][r]);
+      if (out_f32) ((float*)out)[at + nt * 16] = acc[nt][r] * gm;
+      else ((bf16*)out)[at + nt * 16] = static_cast<bf16>(acc[nt][r] * gm);
     }
   }
 }
 
 extern "C" int ms_head_gemm_bf16(const void* x, int ldx, const void* w, void* out, int ldc, int out_stride, int col0, int out_f32,
-                                 int M, int H, int N, int K, hipStream_t st) {
+                                 int M, int H, int N, int K, const float* gate, int gate_ld, int gate_col, hipStream_t st) {
   if (M <= 0 || H <= 0 || N <= 0) return MS_OK;
   if (K <= 0 || ldx < H * K || out_stride < col0 + N || ldc < H * out_stride || col0 < 0 || H > 65535 || (N + 63) / 64 > 65535)
     return MS_BAD_ARG;
+  if (gate && (gate_col < 0 || gate_ld < gate_col + H)) return MS_BAD_ARG;
   if (K % 8 || ldx % 8 || ((size_t)x % 16) || ((size_t)w % 16)) return MS_UNSUPPORTED;
   head_gemm_bf16_kernel<<<dim3((M + 63) / 64, (N + 63) / 64, H), 256, 0, st>>>((const bf16*)x, ldx, (const bf16*)w, out, ldc, out_stride,
-                                                                             col0, M, N, K, out_f32);
+                                                                             col0, M, N, K, out_f32, gate, gate_ld, gate_col);
   return launch_status();
 }

@@ -68,7 +68,8 @@ _SIGNATURES = {
                                            _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_float,
                                            _c_void, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_paged_attention_tiled_mfma_wide_chunk": [_c_int, _c_int, _c_int, _c_int, _c_int],
-    "ms_head_gemm_bf16": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_head_gemm_bf16": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int,
+                          _c_int, _c_void],
     "ms_head_gate": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_activate": [_c_void, _c_void, _c_int, _c_ll, _c_int, _c_void],
     "ms_paged_attention_tiled": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
@@ -1249,12 +1250,14 @@ def activate(x: torch.Tensor, activation: str, out_dtype) -> torch.Tensor:
     return out
 
 
-def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_col: int = 0) -> torch.Tensor:
+def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_col: int = 0, gate=None) -> torch.Tensor:
     """A matrix product per head: ``out[:, h * stride + out_col : ... + N] = x[:, h * K : (h + 1) * K] @ weights[h]^T`` with
     ``x [M, H K]``, ``weights [H, N, K]`` and ``out [M, H stride]`` (``stride = out.shape[1] / H >= out_col + N``; the other
     columns of ``out`` stay). bfloat16 weights with ``K`` a multiple of 8: one launch of a matrix-core kernel for all
     heads. float32 weights: the true 32-bit product, one launch per head over strided rows. Other sizes: head by head
-    through contiguous copies."""
+    through contiguous copies. ``gate = (g, col)``: head ``h``'s results of row ``m`` are multiplied by
+    ``sigmoid(g[m, col + h])`` (``g`` float32; ``out_col`` 0 and ``N`` the head's whole stride): in the matrix-core
+    kernel's epilogue, else by ``head_gate_`` behind the products."""
     _dev(x, "x", (F32, BF16), 2)
     _dev(weights, "weights", (F32, BF16), 3)
     _dev(out, "out", (F32, BF16), 2)
@@ -1266,6 +1269,14 @@ def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_c
         return out
     stride = out.shape[1] // h
     lib = library()
+    if gate is not None:
+        g, g_col = gate
+        _dev(g, "gate", F32, 2)
+        if g.shape[0] != m or g.shape[1] < g_col + h or out_col != 0 or stride != n:
+            raise ValueError("a gate needs one float32 column per head and products that fill their heads' columns")
+        if not (weights.dtype == BF16 and k % 8 == 0):
+            head_linear(x, weights, out, out_col)
+            return head_gate_(out, g, g_col, h)
     if weights.dtype == F32:
         xa = cast(x, F32)
         for i in range(h):
@@ -1276,7 +1287,9 @@ def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_c
     xa = cast(x, BF16)
     if k % 8 == 0:
         _check(lib.ms_head_gemm_bf16(xa.data_ptr(), h * k, weights.data_ptr(), out.data_ptr(), out.shape[1], stride, int(out_col),
-                                     int(out.dtype == F32), m, h, n, k, _stream()), "head_gemm_bf16")
+                                     int(out.dtype == F32), m, h, n, k, gate[0].data_ptr() if gate is not None else None,
+                                     gate[0].shape[1] if gate is not None else 0, int(gate[1]) if gate is not None else 0, _stream()),
+               "head_gemm_bf16")
         return out
     for i in range(h):
         y = linear(xa[:, i * k : (i + 1) * k].contiguous(), weights[i], out_dtype=out.dtype)

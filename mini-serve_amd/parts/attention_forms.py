@@ -229,9 +229,7 @@ class LatentAttention(Mixer):
         a = ops.paged_attention(q_full, cache.k, cache.v, cache.block_table, batch, self.heads, 1, self.key_dim, self.scale,
                                 self.window, self.latent_dim, sinks=self.sink)
         o = torch.empty((x.shape[0], self.heads * self.value_dim), dtype=self.rt.dtype, device=x.device)
-        ops.head_linear(a, self.uv, o, 0)
-        if self.gate:
-            ops.head_gate_(o, x32, self.g_col, self.heads)
+        ops.head_linear(a, self.uv, o, 0, gate=(x32, self.g_col) if self.gate else None)
         return ops.linear(o, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:

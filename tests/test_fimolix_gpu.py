@@ -129,6 +129,12 @@ def test_product_per_head(heads, k, n, stride, col, dtype):
         for h in range(heads):
             want[:, h, col : col + n] = xr[:, h * k : (h + 1) * k] @ wr[h].T
         close(out, want.reshape(m, -1), dtype, f"{m} rows", tol=2e-5 if dtype == torch.float32 else 8e-3)
+        if col == 0 and stride == n:  # with a gate per head in the product's epilogue (or behind it)
+            g = rng.normal(size=(m, heads + 3)) * 2
+            gated = torch.empty((m, heads * n), dtype=dtype, device=DEV)
+            ops().head_linear(dev(x, dtype), dev(w, dtype), gated, 0, gate=(dev(g), 2))
+            close(gated, (want * F.sigmoid(g[:, 2 : 2 + heads])[:, :, None]).reshape(m, -1), dtype, f"{m} rows, gated",
+                  tol=2e-5 if dtype == torch.float32 else 8e-3)
 
 
 def conv_setup(rng, gq, gk, hv, d, dv, taps, dtype, norm=True):
