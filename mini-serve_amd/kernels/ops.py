@@ -687,7 +687,10 @@ def paged_attention(qkv, k_cache, v_cache, block_table, batch, num_heads, num_kv
     other head sizes or page sizes, values of another size than the keys, kept first keys, or
     ``exact_weights``: softmax weights that must meet the values unrounded) runs the generic kernel.
 
-    Options that only the generic kernel knows (float32 arithmetic throughout, head sizes up to 1024):
+    Options of the generic kernel (float32 arithmetic throughout, head sizes up to 1024) and of the second tiled
+    matrix-core kernel (bfloat16 storage, 16-token pages, key sizes that are multiples of 32 and value sizes that are
+    multiples of 16, up to 64 query heads per key head; softmax weights unrounded; rows of several tokens, and steps of
+    single tokens only, whose keys are shared among a block's waves and among blocks):
     ``softcap > 0`` bounds a scaled score ``s`` to ``softcap * tanh(s / softcap)``; ``sinks`` (float32 ``[Hq]``) adds
     ``exp(sinks[h])`` to head ``h``'s softmax denominator; ``value_share = n`` lets ``n`` consecutive key heads weigh
     the same value head (``v_cache`` then has ``Hkv / n`` heads); ``values_in_keys`` takes the first ``Dv`` elements
