@@ -700,18 +700,41 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
     const int* __restrict__ block_table, int table_width, const int* __restrict__ tile_first,
     const int* __restrict__ tile_count, const int* __restrict__ token_row, const int* __restrict__ pos, bf16* __restrict__ out,
     float* __restrict__ out32, int Hq, int Hkv, int D, int Dv, float scale, int window, int keep_first, float softcap,
-    const float* __restrict__ sinks, int value_share, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const float* __restrict__ sinks, int value_share, int splits, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int xcd_combos, int n_tiles) {
   constexpr int PS = WAVE + 4;  // floats between a wave's rows of weights
   __shared__ __attribute__((aligned(16))) float Pw[4][16][PS];
   __shared__ float Mo[SPLIT ? 4 : 1][SPLIT ? 16 : 1][SPLIT ? DVC : 1];  // SPLIT: the waves' outputs, maxima and sums meet here
   __shared__ float Mml[SPLIT ? 4 : 1][16][2];
   extern __shared__ __attribute__((aligned(16))) bf16 Ks[];  // not SPLIT: the tile's keys, [64][D + 8]
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
+  // Which tile, key head and run of values the block owns. xcd_combos > 0 (not SPLIT, a one-dimensional grid): blocks go
+  // to the chip's eight XCDs in turn, and every (key head, run of values) pair is given to XCDs of its own, so that an
+  // XCD's L2 holds the keys and values of its pairs only: a prompt's tiles all walk the same keys, and what they walk
+  // should stay in the 4 MB next to them.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if (!SPLIT && xcd_combos > 0) {
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8, runs_v = Dv / DVC;
+    int combo, t;
+    if (xcd_combos <= 8) {
+      const int per = 8 / xcd_combos;  // XCDs that share a pair take its tiles in turn
+      combo = xcd / per;
+      t = slot * per + xcd % per;
+    } else {
+      const int groups = xcd_combos / 8;  // pairs an XCD owns
+      combo = xcd + 8 * (slot % groups);
+      t = slot / groups;
+    }
+    if (t >= n_tiles) return;
+    bx = t;
+    by = combo / runs_v;
+    bz = combo % runs_v;
+  }
   // SPLIT: a tile is one token, and a block owns up to 16 of a key head's query heads (blockIdx.y names key head and run)
-  const int g = Hq / Hkv, e0 = blockIdx.z * DVC, runs16 = SPLIT ? (g + 15) / 16 : 1;
-  const int kvh = blockIdx.y / runs16, hoff = (blockIdx.y % runs16) * 16;
+  const int g = Hq / Hkv, e0 = bz * DVC, runs16 = SPLIT ? (g + 15) / 16 : 1;
+  const int kvh = by / runs16, hoff = (by % runs16) * 16;
   const int Hv = Hkv / value_share, vh = kvh / value_share;
-  const int tile = SPLIT ? blockIdx.x / splits : blockIdx.x, split = SPLIT ? blockIdx.x % splits : 0;
+  const int tile = SPLIT ? bx / splits : bx, split = SPLIT ? bx % splits : 0;
   const int first = tile_first[tile], count = SPLIT ? 1 : tile_count[tile];
   const int rows = SPLIT ? (g - hoff < 16 ? g - hoff : 16) : count * g;
   const int rb = SPLIT ? 0 : wave * 16;  // SPLIT: every wave holds the tile's (at most 16) rows and takes every fourth key tile
@@ -1078,12 +1101,24 @@ extern "C" int ms_paged_attention_tiled_mfma_wide(const void* q, int q_stride, c
   const size_t key_lds = (size_t)WAVE * (D + 8) * sizeof(bf16);
   if (splits == 0 && key_lds > 140 * 1024) return MS_UNSUPPORTED;
   dim3 grid(splits > 0 ? tiles * splits : tiles, splits > 0 ? Hkv * runs16 : Hkv, Dv / chunk);
+  // rows of several tokens: (key head, run of values) pairs on XCDs of their own where their number divides 8 or is a
+  // multiple of it (a one-dimensional grid of 8 x slots blocks; see the kernel)
+  int combos = 0;
+  if (splits == 0) {
+    const long c = (long)Hkv * (Dv / chunk);
+    if (c <= 8 ? 8 % c == 0 : c % 8 == 0) {
+      combos = (int)c;
+      const long blocks = c <= 8 ? 8L * ((tiles + 8 / c - 1) / (8 / c)) : (long)tiles * c;
+      if (blocks > 0x7fffffffL) combos = 0;
+      else grid = dim3((unsigned)blocks, 1, 1);
+    }
+  }
   const int nq = D <= 128 ? 4 : D <= 576 ? 18 : 0;  // 32-element runs of a query the kernel keeps in registers
 #define TWQ(CC, SP, QQ)                                                                                                        \
   paged_attention_tiled_mfma_wide_kernel<CC, SP, QQ><<<grid, 256, SP ? 0 : key_lds, st>>>(                                     \
       (const bf16*)q, q_stride, (const bf16*)kc, (const bf16*)vc, block_table, table_width, tile_first, tile_count, token_row, pos, \
       o16, o32, Hq, Hkv, D, Dv, scale, window, keep_first, softcap, sinks, value_share, SP ? splits : 1, SP ? part_o : nullptr,     \
-      SP ? part_ml : nullptr)
+      SP ? part_ml : nullptr, combos, tiles)
 #define TW(CC)                                                                                                                 \
   do {                                                                                                                         \
     if (splits > 0) {                                                                                                          \
