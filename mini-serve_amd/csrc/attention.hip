@@ -848,12 +848,15 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
       // run's under way while this one is multiplied.
       __syncthreads();  // the tile before has been read
       const int ld = D + 8;
+      // 16-byte loads of the tile a thread has under way at once: all of them where the queries' registers say how many
+      // there are at most (keys of 128 elements: 4 a thread, of 576: 18), else 6 at a time
+      constexpr int STAGE_BATCH = NQ == 4 ? 4 : NQ == 18 ? 18 : 6;
       int jj = stage_key, c = stage_run;  // thread's first 16-byte run; the next is 256 runs on (no division in the loop)
-      for (int i0 = threadIdx.x; i0 < WAVE * key_runs; i0 += 6 * 256) {
-        uint4 got[6];
-        int at[6];
+      for (int i0 = threadIdx.x; i0 < WAVE * key_runs; i0 += STAGE_BATCH * 256) {
+        uint4 got[STAGE_BATCH];
+        int at[STAGE_BATCH];
 #pragma unroll
-        for (int u = 0; u < 6; ++u) {
+        for (int u = 0; u < STAGE_BATCH; ++u) {
           const int j = j0 + jj;
           const int page = jj < 16 ? pg4.x : jj < 32 ? pg4.y : jj < 48 ? pg4.z : pg4.w;
           at[u] = i0 + u * 256 < WAVE * key_runs ? jj * ld + c * 8 : -1;
@@ -868,7 +871,7 @@ __global__ __launch_bounds__(256) void paged_attention_tiled_mfma_wide_kernel(
           }
         }
 #pragma unroll
-        for (int u = 0; u < 6; ++u)
+        for (int u = 0; u < STAGE_BATCH; ++u)
           if (at[u] >= 0) *reinterpret_cast<uint4*>(Ks + at[u]) = got[u];
       }
       bf16x8 qn = (NQ == 0 && qp && chunks > 0) ? load_bf16x8(qp) : zero_bf16x8();
